@@ -1,0 +1,254 @@
+// Token -> expert dispatch: LDS histogram, prefix sum, stable permutation, and
+// the copy of the routed rows into per-expert segments.  Replaces
+// count_expert_assignments_kernel, exclusive_scan_small_kernel and
+// build_expert_assignments_kernel (utility/utility.cpp:1058-1106, :758-777),
+// whose order inside an expert segment is the order global atomics happen to
+// resolve in (utility.cpp:1101).  Here the order is fixed: inside a segment
+// assignments are sorted by token index, then by slot.  No global atomics.
+#include "moe_internal.h"
+
+namespace moe {
+
+constexpr int kDispThreads = 256;  // tokens per workgroup in count / scatter
+
+// Pass 1: per-workgroup histogram of expert ids over active rows.  Also resets
+// rowmap and perm to -1 (a fill kernel rather than a memset so that the call
+// sequence can be captured in a graph).
+__global__ __launch_bounds__(kDispThreads) void dispatch_count_kernel(
+    const int *__restrict__ topk_i, const int *__restrict__ pos, int T, int E,
+    int *__restrict__ blk_counts, int *__restrict__ rowmap, int a_pad_cap, int *__restrict__ perm) {
+  __shared__ int hist[256];
+  const int tid = threadIdx.x;
+  hist[tid] = 0;
+  __syncthreads();
+  const int t = blockIdx.x * kDispThreads + tid;
+  if (t < T && !(pos && pos[t] < 0)) {
+    const int4 ids = *reinterpret_cast<const int4 *>(topk_i + (size_t)t * kTopK);
+    const int id[kTopK] = {ids.x, ids.y, ids.z, ids.w};
+#pragma unroll
+    for (int k = 0; k < kTopK; k++) {
+      if (id[k] >= 0 && id[k] < E) atomicAdd(&hist[id[k]], 1);
+    }
+  }
+  __syncthreads();
+  if (tid < E) blk_counts[(size_t)blockIdx.x * E + tid] = hist[tid];
+  for (int i = blockIdx.x * kDispThreads + tid; i < a_pad_cap; i += gridDim.x * kDispThreads)
+    rowmap[i] = -1;
+  for (int i = blockIdx.x * kDispThreads + tid; i < T * kTopK; i += gridDim.x * kDispThreads)
+    perm[i] = -1;
+}
+
+__device__ __forceinline__ int block_exclusive_scan_256(int v, int *buf, int tid, int *total) {
+  buf[tid] = v;
+  __syncthreads();
+#pragma unroll
+  for (int off = 1; off < 256; off <<= 1) {
+    const int add = tid >= off ? buf[tid - off] : 0;
+    __syncthreads();
+    buf[tid] += add;
+    __syncthreads();
+  }
+  const int incl = buf[tid];
+  *total = buf[255];
+  __syncthreads();
+  return incl - v;
+}
+
+// Pass 2 (one workgroup): turns the per-workgroup counts into exclusive bases,
+// and builds per-expert offsets and the row-tile plan of the grouped GEMMs.
+// An expert with M rows gets n_mt = ceil(M / 256) tiles of equal height
+// 64 * rb, rb = ceil(M / (64 * n_mt)) in 1..4; its segment in the padded row
+// space is n_mt * 64 * rb rows long, so tiles never overlap the next expert.
+__global__ __launch_bounds__(256) void dispatch_scan_kernel(int *__restrict__ blk_counts, int n_blk,
+                                                           int E, int *__restrict__ offsets,
+                                                           ExpertInfo *__restrict__ info,
+                                                           int *__restrict__ totals) {
+  __shared__ int buf[256];
+  const int e = threadIdx.x;
+  int count = 0;
+  if (e < E) {
+    for (int b = 0; b < n_blk; b++) {
+      const int c = blk_counts[(size_t)b * E + e];
+      blk_counts[(size_t)b * E + e] = count;
+      count += c;
+    }
+  }
+  const int n_mt = (count + kTileRows - 1) / kTileRows;
+  const int rb = n_mt ? (count + kTileGran * n_mt - 1) / (kTileGran * n_mt) : 0;
+  const int padded = n_mt * rb * kTileGran;
+  int tot_count, tot_pad, tot_mt;
+  const int ex_count = block_exclusive_scan_256(count, buf, e, &tot_count);
+  const int ex_pad = block_exclusive_scan_256(padded, buf, e, &tot_pad);
+  const int ex_mt = block_exclusive_scan_256(n_mt, buf, e, &tot_mt);
+  if (e < E) {
+    offsets[e] = ex_count;
+    ExpertInfo inf;
+    inf.row0 = ex_pad;
+    inf.rows = count;
+    inf.n_mt = n_mt;
+    inf.rb = rb;
+    inf.tile_base = ex_mt;
+    inf.pad_[0] = inf.pad_[1] = inf.pad_[2] = 0;
+    info[e] = inf;
+  }
+  if (e == 0) {
+    offsets[E] = tot_count;
+    totals[0] = tot_mt;
+    totals[1] = tot_pad;
+    totals[2] = tot_count;
+    totals[3] = 0;
+  }
+}
+
+// Pass 3: rank of every assignment inside its expert = (assignments of lower
+// workgroups) + (lower waves of this workgroup) + (lower lanes of this wave)
+// + (lower slots of this token), all for the same expert.
+__global__ __launch_bounds__(kDispThreads) void dispatch_scatter_kernel(
+    const int *__restrict__ topk_i, const int *__restrict__ pos, int T, int E,
+    const int *__restrict__ blk_base, const int *__restrict__ offsets,
+    const ExpertInfo *__restrict__ info, int *__restrict__ perm, int *__restrict__ rowmap,
+    int *__restrict__ inv) {
+  __shared__ int wave_cnt[kDispThreads / 64][256];
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int w = tid >> 6;
+  const int t = blockIdx.x * kDispThreads + tid;
+  int id[kTopK] = {-1, -1, -1, -1};
+  if (t < T && !(pos && pos[t] < 0)) {
+    const int4 ids = *reinterpret_cast<const int4 *>(topk_i + (size_t)t * kTopK);
+    id[0] = ids.x; id[1] = ids.y; id[2] = ids.z; id[3] = ids.w;
+#pragma unroll
+    for (int k = 0; k < kTopK; k++)
+      if (id[k] >= E) id[k] = -1;
+  }
+  const unsigned long long lt = (1ull << lane) - 1ull;
+  int rank[kTopK] = {0, 0, 0, 0};
+  for (int e = 0; e < E; e++) {
+    int below = 0;  // matches in lower lanes
+    int total = 0;
+    int mine = 0;   // matches in lower slots of this lane
+#pragma unroll
+    for (int k = 0; k < kTopK; k++) {
+      const bool hit = id[k] == e;
+      const unsigned long long m = __ballot(hit);
+      below += __popcll(m & lt);
+      total += __popcll(m);
+      if (hit) rank[k] = mine;  // completed below once `below` is final
+      mine += hit ? 1 : 0;
+    }
+#pragma unroll
+    for (int k = 0; k < kTopK; k++)
+      if (id[k] == e) rank[k] += below;
+    if (lane == 0) wave_cnt[w][e] = total;
+  }
+  __syncthreads();
+  if (t >= T) return;
+  int out_inv[kTopK];
+#pragma unroll
+  for (int k = 0; k < kTopK; k++) {
+    const int e = id[k];
+    const int a = t * kTopK + k;
+    if (e < 0) { out_inv[k] = -1; continue; }
+    int r = blk_base[(size_t)blockIdx.x * E + e] + rank[k];
+    for (int ww = 0; ww < w; ww++) r += wave_cnt[ww][e];
+    const int prow = info[e].row0 + r;
+    perm[offsets[e] + r] = a;
+    rowmap[prow] = a;
+    out_inv[k] = prow;
+  }
+  *reinterpret_cast<int4 *>(inv + (size_t)t * kTopK) =
+      make_int4(out_inv[0], out_inv[1], out_inv[2], out_inv[3]);
+}
+
+// Copies the routed rows of x into the padded per-expert row space, already in
+// the A-operand fragment order of v_mfma_f32_32x32x16_bf16: fragment
+// (row block rb, k block kb) is 64 lanes x 16 bytes, lane l = row rb*32 + l%32,
+// k = 16*kb + 8*(l/32) .. +7.  Padding rows are zero.  One wave writes four
+// consecutive k blocks (4 KB) of one row block.
+__global__ __launch_bounds__(256) void gather_rows_kernel(const uint16_t *__restrict__ x,
+                                                         const int *__restrict__ rowmap,
+                                                         const int *__restrict__ totals,
+                                                         uint4 *__restrict__ xg, int H) {
+  const int rb = blockIdx.y;
+  if (rb * kRowBlock >= totals[1]) return;
+  const int lane = threadIdx.x & 63;
+  const int grp = blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int kb_total = H / kFragK;
+  if (grp * 4 >= kb_total) return;
+  const int a = rowmap[rb * kRowBlock + (lane & 31)];
+  const uint16_t *src = a >= 0 ? x + (size_t)(a / kTopK) * H + grp * 64 + 8 * (lane >> 5) : nullptr;
+  uint4 *dst = xg + ((size_t)rb * kb_total + grp * 4) * 64 + lane;
+#pragma unroll
+  for (int kk = 0; kk < 4; kk++) {
+    uint4 v = make_uint4(0, 0, 0, 0);
+    if (src) v = *reinterpret_cast<const uint4 *>(src + kk * kFragK);
+    dst[kk * 64] = v;
+  }
+}
+
+// out[t,:] (+)= sum_k topk_v[t,k] * y[inv[t,k],:], slots added in order 0..3
+// (descending router score, as reduce_mlp2_slots_kernel does,
+// utility/utility.cpp:701-726).  Every token owns its K rows of y, so there
+// are no atomics.
+__global__ __launch_bounds__(256) void combine_kernel(const float *__restrict__ y,
+                                                     const int *__restrict__ inv,
+                                                     const float *__restrict__ topk_v,
+                                                     const int *__restrict__ pos,
+                                                     float *__restrict__ out, int H, int accumulate) {
+  const int t = blockIdx.x;
+  const bool active = !(pos && pos[t] < 0);
+  if (!active && accumulate) return;
+  int p[kTopK] = {-1, -1, -1, -1};
+  float w[kTopK] = {0.f, 0.f, 0.f, 0.f};
+  if (active) {
+    const int4 pi = *reinterpret_cast<const int4 *>(inv + (size_t)t * kTopK);
+    const float4 wv = *reinterpret_cast<const float4 *>(topk_v + (size_t)t * kTopK);
+    p[0] = pi.x; p[1] = pi.y; p[2] = pi.z; p[3] = pi.w;
+    w[0] = wv.x; w[1] = wv.y; w[2] = wv.z; w[3] = wv.w;
+  }
+  float4 *o = reinterpret_cast<float4 *>(out + (size_t)t * H);
+  for (int c = threadIdx.x; c < H / 4; c += 256) {
+    float4 s = accumulate ? o[c] : make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+    for (int k = 0; k < kTopK; k++) {
+      if (p[k] >= 0) {
+        const float4 v = reinterpret_cast<const float4 *>(y + (size_t)p[k] * H)[c];
+        s.x += w[k] * v.x; s.y += w[k] * v.y; s.z += w[k] * v.z; s.w += w[k] * v.w;
+      }
+    }
+    o[c] = s;
+  }
+}
+
+hipError_t launch_dispatch(const int *topk_i, const int *pos, int T, int E, const DispatchBuffers &d,
+                           hipStream_t s) {
+  const int n_blk = (T + kDispThreads - 1) / kDispThreads;
+  // Rows of the padded space this batch can reach: sum over experts of
+  // n_mt * 64 * rb < 1.25 * A + 64 * E.
+  const long long A = (long long)T * kTopK;
+  const long long reach = A + A / 4 + (long long)kTileGran * E;
+  const int fill_rows = (int)(reach < d.a_pad_cap ? reach : d.a_pad_cap);
+  dispatch_count_kernel<<<n_blk, kDispThreads, 0, s>>>(topk_i, pos, T, E, d.blk_counts, d.rowmap,
+                                                       fill_rows, d.perm);
+  dispatch_scan_kernel<<<1, 256, 0, s>>>(d.blk_counts, n_blk, E, d.offsets, d.info, d.totals);
+  dispatch_scatter_kernel<<<n_blk, kDispThreads, 0, s>>>(topk_i, pos, T, E, d.blk_counts, d.offsets,
+                                                         d.info, d.perm, d.rowmap, d.inv);
+  return hipGetLastError();
+}
+
+hipError_t launch_gather(const uint16_t *x, const DispatchBuffers &d, uint16_t *xg, int T, int H,
+                         int rb_cap, hipStream_t s) {
+  (void)T;
+  const int groups = H / 64;
+  dim3 grid((groups + 3) / 4, rb_cap);
+  gather_rows_kernel<<<grid, 256, 0, s>>>(x, d.rowmap, d.totals, reinterpret_cast<uint4 *>(xg), H);
+  return hipGetLastError();
+}
+
+hipError_t launch_combine(const float *y, const int *inv, const float *topk_v, const int *pos,
+                          float *out, int T, int H, int accumulate, hipStream_t s) {
+  combine_kernel<<<T, 256, 0, s>>>(y, inv, topk_v, pos, out, H, accumulate);
+  return hipGetLastError();
+}
+
+}  // namespace moe

@@ -1,0 +1,453 @@
+// Host side of the C-ABI (include/moe_abi.h): handle, weight ingest, stage
+// orchestration, per-stage event timing.  Plays the role of the host code of
+// getp-csrc/expert.cpp (init :709-1174, forward :1366-1607, cleanup :1234-1364)
+// and of the local MoE path in getp_run.cpp:697-845, for one GPU.
+#include <stdarg.h>
+#include <stdio.h>
+#include <string.h>
+
+#include <new>
+#include <vector>
+
+#include "moe_internal.h"
+
+using namespace moe;
+
+namespace {
+
+thread_local char g_err[512] = "";
+
+int fail(int code, const char *fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+#define HIP_TRY(call)                                                                       \
+  do {                                                                                      \
+    hipError_t e_ = (call);                                                                 \
+    if (e_ != hipSuccess)                                                                   \
+      return fail(MOE_ERR_HIP, "%s failed: %s (%s:%d)", #call, hipGetErrorString(e_), __FILE__, \
+                  __LINE__);                                                                \
+  } while (0)
+
+int next_router_pad(int E) {
+  for (int p = 16; p <= 256; p <<= 1)
+    if (E <= p) return p;
+  return -1;
+}
+
+constexpr int kMaxProfileCalls = 256;
+
+}  // namespace
+
+struct moe_handle {
+  moe_config cfg{};
+  int device = 0;
+  int E_pad = 0;
+  std::vector<LayerWeights> layers;
+  size_t layer_bytes = 0;
+  size_t ws_bytes = 0;
+
+  // routing produced by the router stage (or copied from the caller)
+  int *topk_i = nullptr;
+  float *topk_v = nullptr;
+  // dispatch
+  DispatchBuffers disp{};
+  int a_cap = 0;      // max assignments
+  int a_pad_cap = 0;  // max padded rows
+  int n_blk_cap = 0;
+  // expert pipeline
+  uint16_t *xg = nullptr;   // gathered rows, bf16 fragments
+  uint16_t *act = nullptr;  // SwiGLU output, bf16 fragments
+  float *y = nullptr;       // down output [a_pad_cap, H]
+
+  // profiling
+  std::vector<hipEvent_t> events;  // kMaxProfileCalls * (MOE_NUM_STAGES + 1)
+  int prof_armed = 0;              // calls still to record
+  int prof_recorded = 0;
+};
+
+namespace {
+
+template <typename T>
+int dev_alloc(moe_handle *h, T **p, size_t count, bool workspace) {
+  void *q = nullptr;
+  const size_t bytes = count * sizeof(T);
+  hipError_t e = hipMalloc(&q, bytes ? bytes : 1);
+  if (e != hipSuccess)
+    return fail(MOE_ERR_HIP, "hipMalloc(%zu bytes) failed: %s", bytes, hipGetErrorString(e));
+  *p = static_cast<T *>(q);
+  if (workspace) h->ws_bytes += bytes;
+  return MOE_OK;
+}
+
+int check_forward_args(moe_handle *h, int layer, const void *x, int n_tokens, const void *out) {
+  if (!h) return fail(MOE_ERR_BAD_ARG, "null handle");
+  if (layer < 0 || layer >= h->cfg.layers)
+    return fail(MOE_ERR_BAD_ARG, "layer %d out of range [0,%d)", layer, h->cfg.layers);
+  if (n_tokens < 0) return fail(MOE_ERR_BAD_ARG, "n_tokens %d is negative", n_tokens);
+  if (n_tokens > h->cfg.max_tokens)
+    return fail(MOE_ERR_CAPACITY, "n_tokens %d exceeds max_tokens %d", n_tokens, h->cfg.max_tokens);
+  if (n_tokens > 0 && (!x || !out)) return fail(MOE_ERR_BAD_ARG, "null device pointer");
+  if (!h->layers[layer].uploaded)
+    return fail(MOE_ERR_STATE, "layer %d has no weights (moe_upload_layer not called)", layer);
+  return MOE_OK;
+}
+
+struct StageTimer {
+  moe_handle *h;
+  hipStream_t s;
+  hipEvent_t *ev = nullptr;
+  StageTimer(moe_handle *h_, hipStream_t s_) : h(h_), s(s_) {
+    if (h->prof_armed > 0 && h->prof_recorded < kMaxProfileCalls && !h->events.empty())
+      ev = &h->events[(size_t)h->prof_recorded * (MOE_NUM_STAGES + 1)];
+  }
+  hipError_t mark(int boundary) {  // boundary i = start of stage i; MOE_NUM_STAGES = end
+    return ev ? hipEventRecord(ev[boundary], s) : hipSuccess;
+  }
+  void done() {
+    if (ev) {
+      h->prof_recorded++;
+      h->prof_armed--;
+    }
+  }
+};
+
+int run_experts(moe_handle *h, int layer, const uint16_t *x, const int *pos, const int *topk_i,
+                const float *topk_v, int T, float *out, int accumulate, hipStream_t s,
+                StageTimer &tm) {
+  const moe_config &c = h->cfg;
+  const LayerWeights &lw = h->layers[layer];
+  const int A = T * kTopK;
+  const int mt_cap = A / kTileRows + c.experts;
+  const int rb_cap = (A + A / 4 + kTileGran * c.experts + kRowBlock - 1) / kRowBlock;
+  HIP_TRY(tm.mark(MOE_STAGE_DISPATCH));
+  HIP_TRY(launch_dispatch(topk_i, pos, T, c.experts, h->disp, s));
+  HIP_TRY(tm.mark(MOE_STAGE_GATHER));
+  HIP_TRY(launch_gather(x, h->disp, h->xg, T, c.hidden, rb_cap, s));
+  HIP_TRY(tm.mark(MOE_STAGE_GATE_UP));
+  HIP_TRY(launch_gate_up(h->xg, lw.w1, lw.b1g, lw.b1u, h->disp, h->act, c.hidden, c.inter,
+                         c.experts, c.swiglu_limit, mt_cap, s));
+  HIP_TRY(tm.mark(MOE_STAGE_DOWN));
+  HIP_TRY(launch_down(h->act, lw.w2, lw.b2, h->disp, h->y, c.hidden, c.inter, c.experts, mt_cap, s));
+  HIP_TRY(tm.mark(MOE_STAGE_COMBINE));
+  HIP_TRY(launch_combine(h->y, h->disp.inv, topk_v, pos, out, T, c.hidden, accumulate, s));
+  HIP_TRY(tm.mark(MOE_NUM_STAGES));
+  return MOE_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+const char *moe_last_error(void) { return g_err; }
+const char *moe_version(void) { return "mi355-moe 0.1 (gfx950)"; }
+
+int moe_create(const moe_config *cfg, moe_handle **out) {
+  if (!cfg || !out) return fail(MOE_ERR_BAD_ARG, "null argument");
+  *out = nullptr;
+  if (cfg->topk != kTopK)
+    return fail(MOE_ERR_UNSUPPORTED, "topk %d unsupported (kernels are built for 4)", cfg->topk);
+  if (cfg->hidden <= 0 || cfg->hidden % 64 || cfg->inter <= 0 || cfg->inter % 64)
+    return fail(MOE_ERR_UNSUPPORTED, "hidden %d / inter %d must be positive multiples of 64",
+                cfg->hidden, cfg->inter);
+  if (cfg->experts < kTopK || cfg->experts > 256)
+    return fail(MOE_ERR_UNSUPPORTED, "experts %d outside [4,256]", cfg->experts);
+  if (cfg->layers <= 0 || cfg->max_tokens <= 0)
+    return fail(MOE_ERR_BAD_ARG, "layers %d / max_tokens %d must be positive", cfg->layers,
+                cfg->max_tokens);
+  if ((long long)cfg->max_tokens * kTopK > (1ll << 28))
+    return fail(MOE_ERR_UNSUPPORTED, "max_tokens %d too large", cfg->max_tokens);
+  if (!(cfg->swiglu_limit > 0.f)) return fail(MOE_ERR_BAD_ARG, "swiglu_limit must be positive");
+
+  moe_handle *h = new (std::nothrow) moe_handle();
+  if (!h) return fail(MOE_ERR_BAD_ARG, "out of host memory");
+  h->cfg = *cfg;
+  h->E_pad = next_router_pad(cfg->experts);
+  hipError_t e = hipGetDevice(&h->device);
+  if (e != hipSuccess) {
+    delete h;
+    return fail(MOE_ERR_HIP, "hipGetDevice failed: %s", hipGetErrorString(e));
+  }
+  h->layers.resize(cfg->layers);
+
+  const int E = cfg->experts, H = cfg->hidden, IM = cfg->inter, T = cfg->max_tokens;
+  h->a_cap = T * kTopK;
+  h->a_pad_cap = ((h->a_cap + h->a_cap / 4 + kTileGran * E + kTileGran - 1) / kTileGran) * kTileGran;
+  h->n_blk_cap = (T + 255) / 256;
+  int rc = MOE_OK;
+#define ALLOC(ptr, count)                                   \
+  if (rc == MOE_OK) rc = dev_alloc(h, &(ptr), (count), true)
+  ALLOC(h->topk_i, (size_t)h->a_cap);
+  ALLOC(h->topk_v, (size_t)h->a_cap);
+  ALLOC(h->disp.blk_counts, (size_t)h->n_blk_cap * E);
+  ALLOC(h->disp.offsets, (size_t)E + 1);
+  ALLOC(h->disp.perm, (size_t)h->a_cap);
+  ALLOC(h->disp.rowmap, (size_t)h->a_pad_cap);
+  ALLOC(h->disp.inv, (size_t)h->a_cap);
+  ALLOC(h->disp.info, (size_t)E);
+  ALLOC(h->disp.totals, (size_t)4);
+  ALLOC(h->xg, (size_t)h->a_pad_cap * H);
+  ALLOC(h->act, (size_t)h->a_pad_cap * IM);
+  ALLOC(h->y, (size_t)h->a_pad_cap * H);
+#undef ALLOC
+  h->disp.a_pad_cap = h->a_pad_cap;
+  if (rc != MOE_OK) {
+    moe_destroy(h);
+    return rc;
+  }
+  h->layer_bytes = (size_t)h->E_pad * H * 8 + (size_t)h->E_pad * 4 +
+                   (size_t)E * 2 * IM * H * 2 + (size_t)E * 2 * IM * 4 +
+                   (size_t)E * H * IM * 2 + (size_t)E * H * 4;
+  *out = h;
+  return MOE_OK;
+}
+
+int moe_destroy(moe_handle *h) {
+  if (!h) return MOE_OK;
+  for (auto &lw : h->layers) {
+    (void)hipFree(lw.wr); (void)hipFree(lw.br); (void)hipFree(lw.w1); (void)hipFree(lw.b1g);
+    (void)hipFree(lw.b1u); (void)hipFree(lw.w2); (void)hipFree(lw.b2);
+  }
+  (void)hipFree(h->topk_i); (void)hipFree(h->topk_v);
+  (void)hipFree(h->disp.blk_counts); (void)hipFree(h->disp.offsets); (void)hipFree(h->disp.perm);
+  (void)hipFree(h->disp.rowmap); (void)hipFree(h->disp.inv); (void)hipFree(h->disp.info); (void)hipFree(h->disp.totals);
+  (void)hipFree(h->xg); (void)hipFree(h->act); (void)hipFree(h->y);
+  for (hipEvent_t ev : h->events) (void)hipEventDestroy(ev);
+  delete h;
+  return MOE_OK;
+}
+
+int moe_upload_layer(moe_handle *h, int layer, const float *w_router, const float *b_router,
+                     const float *w_mlp1, const float *b_mlp1, const float *w_mlp2,
+                     const float *b_mlp2) {
+  if (!h) return fail(MOE_ERR_BAD_ARG, "null handle");
+  if (layer < 0 || layer >= h->cfg.layers)
+    return fail(MOE_ERR_BAD_ARG, "layer %d out of range [0,%d)", layer, h->cfg.layers);
+  if (!w_router || !b_router || !w_mlp1 || !b_mlp1 || !w_mlp2 || !b_mlp2)
+    return fail(MOE_ERR_BAD_ARG, "null weight pointer");
+  const int E = h->cfg.experts, H = h->cfg.hidden, IM = h->cfg.inter, E_pad = h->E_pad;
+  LayerWeights &lw = h->layers[layer];
+  int rc = MOE_OK;
+#define ALLOCW(ptr, count)                                             \
+  if (rc == MOE_OK && !(ptr)) rc = dev_alloc(h, &(ptr), (count), false)
+  ALLOCW(lw.wr, (size_t)E_pad * H);
+  ALLOCW(lw.br, (size_t)E_pad);
+  ALLOCW(lw.w1, (size_t)E * 2 * IM * H);
+  ALLOCW(lw.b1g, (size_t)E * IM);
+  ALLOCW(lw.b1u, (size_t)E * IM);
+  ALLOCW(lw.w2, (size_t)E * H * IM);
+  ALLOCW(lw.b2, (size_t)E * H);
+#undef ALLOCW
+  if (rc != MOE_OK) return rc;
+
+  // fp32 staging for one expert matrix at a time; conversion and re-ordering
+  // run on the GPU (the reference packs on the host, utility.cpp:568-622).
+  const size_t stage_elems = (size_t)2 * IM * H > (size_t)E * H ? (size_t)2 * IM * H : (size_t)E * H;
+  float *stage = nullptr, *stage_b = nullptr;
+  HIP_TRY(hipMalloc(reinterpret_cast<void **>(&stage), stage_elems * sizeof(float)));
+  const size_t bias_elems = (size_t)E * 2 * IM > (size_t)E * H ? (size_t)E * 2 * IM : (size_t)E * H;
+  hipError_t e = hipMalloc(reinterpret_cast<void **>(&stage_b), bias_elems * sizeof(float));
+  if (e != hipSuccess) {
+    (void)hipFree(stage);
+    return fail(MOE_ERR_HIP, "hipMalloc failed: %s", hipGetErrorString(e));
+  }
+  auto body = [&]() -> int {
+    HIP_TRY(hipMemcpy(stage, w_router, (size_t)E * H * sizeof(float), hipMemcpyHostToDevice));
+    HIP_TRY(hipMemcpy(stage_b, b_router, (size_t)E * sizeof(float), hipMemcpyHostToDevice));
+    HIP_TRY(launch_pack_router(stage, stage_b, lw.wr, lw.br, E, E_pad, H, nullptr));
+    HIP_TRY(hipDeviceSynchronize());
+    HIP_TRY(hipMemcpy(stage_b, b_mlp1, (size_t)E * 2 * IM * sizeof(float), hipMemcpyHostToDevice));
+    HIP_TRY(launch_pack_bias(stage_b, lw.b1g, lw.b1u, E * 2 * IM, true, nullptr));
+    HIP_TRY(hipDeviceSynchronize());
+    HIP_TRY(hipMemcpy(stage_b, b_mlp2, (size_t)E * H * sizeof(float), hipMemcpyHostToDevice));
+    HIP_TRY(launch_pack_bias(stage_b, lw.b2, nullptr, E * H, false, nullptr));
+    HIP_TRY(hipDeviceSynchronize());
+    for (int ex = 0; ex < E; ex++) {
+      HIP_TRY(hipMemcpy(stage, w_mlp1 + (size_t)ex * 2 * IM * H, (size_t)2 * IM * H * sizeof(float),
+                        hipMemcpyHostToDevice));
+      HIP_TRY(launch_pack_weight(stage, lw.w1 + (size_t)ex * 2 * IM * H, 2 * IM, H, true, nullptr));
+      HIP_TRY(hipDeviceSynchronize());
+      HIP_TRY(hipMemcpy(stage, w_mlp2 + (size_t)ex * H * IM, (size_t)H * IM * sizeof(float),
+                        hipMemcpyHostToDevice));
+      HIP_TRY(launch_pack_weight(stage, lw.w2 + (size_t)ex * H * IM, H, IM, false, nullptr));
+      HIP_TRY(hipDeviceSynchronize());
+    }
+    return MOE_OK;
+  };
+  rc = body();
+  (void)hipFree(stage);
+  (void)hipFree(stage_b);
+  if (rc == MOE_OK) lw.uploaded = true;
+  return rc;
+}
+
+int moe_router(moe_handle *h, int layer, const uint16_t *x, const int *pos, int n_tokens,
+               float *score, int *topk_i, float *topk_v, void *stream) {
+  int rc = check_forward_args(h, layer, x, n_tokens, topk_i);
+  if (rc != MOE_OK) return rc;
+  if (n_tokens > 0 && !topk_v) return fail(MOE_ERR_BAD_ARG, "null device pointer");
+  if (n_tokens == 0) return MOE_OK;
+  const LayerWeights &lw = h->layers[layer];
+  HIP_TRY(launch_router(x, pos, lw.wr, lw.br, n_tokens, h->cfg.hidden, h->cfg.experts, h->E_pad,
+                        score, topk_i, topk_v, static_cast<hipStream_t>(stream)));
+  return MOE_OK;
+}
+
+int moe_dispatch(moe_handle *h, const int *topk_i, const int *pos, int n_tokens, void *stream) {
+  if (!h) return fail(MOE_ERR_BAD_ARG, "null handle");
+  if (n_tokens < 0) return fail(MOE_ERR_BAD_ARG, "n_tokens %d is negative", n_tokens);
+  if (n_tokens > h->cfg.max_tokens)
+    return fail(MOE_ERR_CAPACITY, "n_tokens %d exceeds max_tokens %d", n_tokens, h->cfg.max_tokens);
+  if (n_tokens > 0 && !topk_i) return fail(MOE_ERR_BAD_ARG, "null device pointer");
+  HIP_TRY(launch_dispatch(topk_i, pos, n_tokens, h->cfg.experts, h->disp,
+                          static_cast<hipStream_t>(stream)));
+  return MOE_OK;
+}
+
+int moe_get_dispatch(moe_handle *h, int *offsets, int *perm, int n_tokens, void *stream) {
+  if (!h) return fail(MOE_ERR_BAD_ARG, "null handle");
+  if (n_tokens < 0 || n_tokens > h->cfg.max_tokens)
+    return fail(MOE_ERR_BAD_ARG, "n_tokens %d out of range", n_tokens);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (offsets)
+    HIP_TRY(hipMemcpyAsync(offsets, h->disp.offsets, ((size_t)h->cfg.experts + 1) * sizeof(int),
+                           hipMemcpyDeviceToDevice, s));
+  if (perm && n_tokens > 0)
+    HIP_TRY(hipMemcpyAsync(perm, h->disp.perm, (size_t)n_tokens * kTopK * sizeof(int),
+                           hipMemcpyDeviceToDevice, s));
+  return MOE_OK;
+}
+
+int moe_experts(moe_handle *h, int layer, const uint16_t *x, const int *pos, const int *topk_i,
+                const float *topk_v, int n_tokens, float *out, int accumulate, void *stream) {
+  int rc = check_forward_args(h, layer, x, n_tokens, out);
+  if (rc != MOE_OK) return rc;
+  if (n_tokens == 0) return MOE_OK;
+  if (!topk_i || !topk_v) return fail(MOE_ERR_BAD_ARG, "null device pointer");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  StageTimer tm(h, s);
+  HIP_TRY(tm.mark(MOE_STAGE_ROUTER));
+  rc = run_experts(h, layer, x, pos, topk_i, topk_v, n_tokens, out, accumulate, s, tm);
+  if (rc == MOE_OK) tm.done();
+  return rc;
+}
+
+int moe_forward(moe_handle *h, int layer, const uint16_t *x, const int *pos, int n_tokens,
+                float *out, int accumulate, void *stream) {
+  int rc = check_forward_args(h, layer, x, n_tokens, out);
+  if (rc != MOE_OK) return rc;
+  if (n_tokens == 0) return MOE_OK;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const LayerWeights &lw = h->layers[layer];
+  StageTimer tm(h, s);
+  HIP_TRY(tm.mark(MOE_STAGE_ROUTER));
+  HIP_TRY(launch_router(x, pos, lw.wr, lw.br, n_tokens, h->cfg.hidden, h->cfg.experts, h->E_pad,
+                        nullptr, h->topk_i, h->topk_v, s));
+  rc = run_experts(h, layer, x, pos, h->topk_i, h->topk_v, n_tokens, out, accumulate, s, tm);
+  if (rc == MOE_OK) tm.done();
+  return rc;
+}
+
+int moe_profile_enable(moe_handle *h, int n_calls) {
+  if (!h) return fail(MOE_ERR_BAD_ARG, "null handle");
+  if (n_calls < 0 || n_calls > kMaxProfileCalls)
+    return fail(MOE_ERR_BAD_ARG, "n_calls %d outside [0,%d]", n_calls, kMaxProfileCalls);
+  if (h->events.empty()) {
+    h->events.resize((size_t)kMaxProfileCalls * (MOE_NUM_STAGES + 1), nullptr);
+    for (auto &ev : h->events) HIP_TRY(hipEventCreate(&ev));
+  }
+  h->prof_armed = n_calls;
+  h->prof_recorded = 0;
+  return MOE_OK;
+}
+
+int moe_profile_read(moe_handle *h, float *ms, int *n_calls) {
+  if (!h || !ms) return fail(MOE_ERR_BAD_ARG, "null argument");
+  if (h->events.empty()) return fail(MOE_ERR_STATE, "profiling was never enabled");
+  double sum[MOE_NUM_STAGES] = {0};
+  for (int c = 0; c < h->prof_recorded; c++) {
+    hipEvent_t *ev = &h->events[(size_t)c * (MOE_NUM_STAGES + 1)];
+    HIP_TRY(hipEventSynchronize(ev[MOE_NUM_STAGES]));
+    for (int st = 0; st < MOE_NUM_STAGES; st++) {
+      float t = 0.f;
+      HIP_TRY(hipEventElapsedTime(&t, ev[st], ev[st + 1]));
+      sum[st] += t;
+    }
+  }
+  for (int st = 0; st < MOE_NUM_STAGES; st++)
+    ms[st] = h->prof_recorded ? (float)(sum[st] / h->prof_recorded) : 0.f;
+  if (n_calls) *n_calls = h->prof_recorded;
+  return MOE_OK;
+}
+
+size_t moe_weight_bytes(const moe_handle *h) { return h ? h->layer_bytes : 0; }
+size_t moe_workspace_bytes(const moe_handle *h) { return h ? h->ws_bytes : 0; }
+
+int moe_dev_alloc(void **ptr, size_t bytes) {
+  if (!ptr) return fail(MOE_ERR_BAD_ARG, "null argument");
+  HIP_TRY(hipMalloc(ptr, bytes ? bytes : 1));
+  return MOE_OK;
+}
+int moe_dev_free(void *ptr) {
+  HIP_TRY(hipFree(ptr));
+  return MOE_OK;
+}
+int moe_dev_upload(void *dst_dev, const void *src_host, size_t bytes) {
+  HIP_TRY(hipMemcpy(dst_dev, src_host, bytes, hipMemcpyHostToDevice));
+  return MOE_OK;
+}
+int moe_dev_download(void *dst_host, const void *src_dev, size_t bytes) {
+  HIP_TRY(hipMemcpy(dst_host, src_dev, bytes, hipMemcpyDeviceToHost));
+  return MOE_OK;
+}
+int moe_dev_memset(void *dst_dev, int value, size_t bytes) {
+  HIP_TRY(hipMemset(dst_dev, value, bytes));
+  return MOE_OK;
+}
+int moe_dev_sync(void) {
+  HIP_TRY(hipDeviceSynchronize());
+  return MOE_OK;
+}
+int moe_dev_count(void) {
+  int n = 0;
+  if (hipGetDeviceCount(&n) != hipSuccess) return 0;
+  return n;
+}
+
+int moe_time_forward(moe_handle *h, int layer, const uint16_t *x, const int *pos, int n_tokens,
+                     float *out, int warmup, int iters, float *total_ms) {
+  if (!total_ms || iters <= 0 || warmup < 0) return fail(MOE_ERR_BAD_ARG, "bad timing arguments");
+  hipStream_t s = nullptr;
+  HIP_TRY(hipStreamCreate(&s));
+  hipEvent_t e0 = nullptr, e1 = nullptr;
+  int rc = MOE_OK;
+  auto body = [&]() -> int {
+    HIP_TRY(hipEventCreate(&e0));
+    HIP_TRY(hipEventCreate(&e1));
+    for (int i = 0; i < warmup; i++) {
+      int r = moe_forward(h, layer, x, pos, n_tokens, out, 0, s);
+      if (r != MOE_OK) return r;
+    }
+    HIP_TRY(hipStreamSynchronize(s));
+    HIP_TRY(hipEventRecord(e0, s));
+    for (int i = 0; i < iters; i++) {
+      int r = moe_forward(h, layer, x, pos, n_tokens, out, 0, s);
+      if (r != MOE_OK) return r;
+    }
+    HIP_TRY(hipEventRecord(e1, s));
+    HIP_TRY(hipEventSynchronize(e1));
+    HIP_TRY(hipEventElapsedTime(total_ms, e0, e1));
+    return MOE_OK;
+  };
+  rc = body();
+  if (e0) (void)hipEventDestroy(e0);
+  if (e1) (void)hipEventDestroy(e1);
+  (void)hipStreamDestroy(s);
+  return rc;
+}
+
+}  // extern "C"

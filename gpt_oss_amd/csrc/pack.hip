@@ -1,0 +1,112 @@
+// Weight ingest: fp32 host layout of the reference (run.cpp:234-247) -> bf16
+// (round to nearest even, as utility.cpp:509/:534/:610 do at upload) in the
+// fragment order the gfx950 MFMA kernels read.  Replaces
+// pack_fp32_to_bf16_matmul (utility/utility.cpp:558-622) and the per-expert
+// host loops of getp_run.cpp:259-293 / expert.cpp:971-1009.
+#include "moe_internal.h"
+
+namespace moe {
+
+__device__ __forceinline__ uint16_t f32_to_bf16_rne(float f) {
+  uint32_t u = __float_as_uint(f);
+  if (~u & 0x7f800000u) {
+    u += 0x7fffu + ((u >> 16) & 1u);
+  } else if (u & 0xffffu) {
+    u |= 0x10000u;
+  }
+  return (uint16_t)(u >> 16);
+}
+
+__device__ __forceinline__ float bf16_round(float f) {
+  return __uint_as_float((uint32_t)f32_to_bf16_rne(f) << 16);
+}
+
+// One fragment = 32 output rows x 16 reduction elements, stored as 64 lanes x
+// 8 bf16: lane l holds row (l % 32), k = 8*(l / 32) .. +7 -- the B-operand
+// register layout of v_mfma_f32_32x32x16_bf16.  Fragments are ordered
+// [row block][k block].  With gate_up set, row block 2p holds the gate rows
+// (source rows 2j) and row block 2p+1 the up rows (source rows 2j+1) of
+// j = 32p .. 32p+31, so that a lane's gate and up accumulators line up.
+__global__ void pack_weight_kernel(const float *__restrict__ src, uint4 *__restrict__ dst, int rows,
+                                   int cols, int gate_up) {
+  const int kb_total = cols / kFragK;
+  const size_t n_chunks = (size_t)(rows / kRowBlock) * kb_total * 64;
+  for (size_t c = (size_t)blockIdx.x * blockDim.x + threadIdx.x; c < n_chunks;
+       c += (size_t)gridDim.x * blockDim.x) {
+    const int lane = (int)(c & 63);
+    const size_t frag = c >> 6;
+    const int kb = (int)(frag % kb_total);
+    const int nb = (int)(frag / kb_total);
+    const int n = lane & 31;
+    const int k0 = kb * kFragK + 8 * (lane >> 5);
+    const int row = gate_up ? 2 * (kRowBlock * (nb >> 1) + n) + (nb & 1) : kRowBlock * nb + n;
+    const float4 *p = reinterpret_cast<const float4 *>(src + (size_t)row * cols + k0);
+    const float4 a = p[0], b = p[1];
+    uint4 o;
+    o.x = f32_to_bf16_rne(a.x) | ((uint32_t)f32_to_bf16_rne(a.y) << 16);
+    o.y = f32_to_bf16_rne(a.z) | ((uint32_t)f32_to_bf16_rne(a.w) << 16);
+    o.z = f32_to_bf16_rne(b.x) | ((uint32_t)f32_to_bf16_rne(b.y) << 16);
+    o.w = f32_to_bf16_rne(b.z) | ((uint32_t)f32_to_bf16_rne(b.w) << 16);
+    dst[c] = o;
+  }
+}
+
+// Router weight as f64 fragments of v_mfma_f64_16x16x4_f64.  Order
+// [expert block of 16][k chunk of 32][lane][s], s = 0..7: lane l holds expert
+// 16*nb + (l % 16) and k = 32*kc + 8*(l / 16) + s.  The s-th MFMA of a chunk
+// multiplies these with the s-th of 8 consecutive activations a lane loaded.
+// Experts beyond E are zero weight with bias -inf, so they are never selected.
+__global__ void pack_router_kernel(const float *__restrict__ w, const float *__restrict__ b,
+                                   double *__restrict__ wr, float *__restrict__ br, int E, int E_pad,
+                                   int H) {
+  const int kc_total = H / 32;
+  const size_t n = (size_t)(E_pad / 16) * kc_total * 64 * 8;
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n;
+       i += (size_t)gridDim.x * blockDim.x) {
+    const int s = (int)(i & 7);
+    const int lane = (int)((i >> 3) & 63);
+    const size_t f = i >> 9;
+    const int kc = (int)(f % kc_total);
+    const int nb = (int)(f / kc_total);
+    const int e = nb * 16 + (lane & 15);
+    const int k = kc * 32 + 8 * (lane >> 4) + s;
+    wr[i] = e < E ? (double)bf16_round(w[(size_t)e * H + k]) : 0.0;
+  }
+  const int t = blockIdx.x * blockDim.x + threadIdx.x;
+  if (t < E_pad) br[t] = t < E ? bf16_round(b[t]) : -INFINITY;
+}
+
+// Biases are kept as fp32 holding bf16-rounded values (the reference keeps
+// them as bf16, expert.cpp:906-930).  deinterleave: src[2j] -> a[j], src[2j+1] -> b[j].
+__global__ void pack_bias_kernel(const float *__restrict__ src, float *__restrict__ a,
+                                 float *__restrict__ b, int n, int deinterleave) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  const float v = bf16_round(src[i]);
+  if (deinterleave) {
+    if (i & 1) b[i >> 1] = v; else a[i >> 1] = v;
+  } else {
+    a[i] = v;
+  }
+}
+
+hipError_t launch_pack_router(const float *w_src, const float *b_src, double *wr, float *br, int E,
+                              int E_pad, int H, hipStream_t s) {
+  pack_router_kernel<<<512, 256, 0, s>>>(w_src, b_src, wr, br, E, E_pad, H);
+  return hipGetLastError();
+}
+
+hipError_t launch_pack_weight(const float *src, uint16_t *dst, int rows, int cols, bool gate_up,
+                              hipStream_t s) {
+  pack_weight_kernel<<<2048, 256, 0, s>>>(src, reinterpret_cast<uint4 *>(dst), rows, cols,
+                                          gate_up ? 1 : 0);
+  return hipGetLastError();
+}
+
+hipError_t launch_pack_bias(const float *src, float *dst_a, float *dst_b, int n, bool deinterleave,
+                            hipStream_t s) {
+  pack_bias_kernel<<<(n + 255) / 256, 256, 0, s>>>(src, dst_a, dst_b, n, deinterleave ? 1 : 0);
+  return hipGetLastError();
+}
+
+}  // namespace moe

@@ -1,0 +1,171 @@
+/*
+ * C-ABI of the MI355X (gfx950) GPT-OSS mixture-of-experts layer.
+ *
+ * Drop-in boundary for the MoE path of pmatuan/gpt-oss in getp mode.  Each
+ * entry point names the reference interface it replaces (file:line relative to
+ * the reference checkout).  All pointers named x / pos / out / topk_* / score
+ * are DEVICE pointers unless stated otherwise; weight pointers given to the
+ * upload calls are HOST pointers in the reference's host layout
+ * (TransformerWeights, run.cpp:67-79, mapped at run.cpp:234-247).
+ *
+ * Every function returns MOE_OK (0) or a negative moe_status; the text of the
+ * last failure on the calling thread is available from moe_last_error().
+ * Nothing here exits the process (the reference's HIP_CHECK does,
+ * common/defines.h:94-102); the host shim turns a non-zero status into that
+ * behaviour.
+ *
+ * A handle belongs to one device and one host thread at a time.  Calls on one
+ * handle are asynchronous on the given stream and never synchronise with the
+ * host; all routing counts and offsets stay on the device.
+ */
+#ifndef MI355_MOE_ABI_H
+#define MI355_MOE_ABI_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct moe_handle moe_handle;
+
+typedef enum {
+  MOE_OK = 0,
+  MOE_ERR_BAD_ARG = -1,     /* null pointer, negative size, unknown layer ... */
+  MOE_ERR_UNSUPPORTED = -2, /* shape outside what the kernels are built for   */
+  MOE_ERR_CAPACITY = -3,    /* n_tokens > max_tokens (getp_run.cpp:532-552)   */
+  MOE_ERR_HIP = -4,         /* a HIP runtime call failed                      */
+  MOE_ERR_STATE = -5        /* layer not uploaded, profiling not enabled ...  */
+} moe_status;
+
+/* Model hyper-parameters of the path: Config fields hidden_dim, n_experts,
+ * experts_per_token, intermediate_dim, n_layers, swiglu_limit (run.cpp:26-46).
+ * max_tokens replaces MAX_BATCH_SIZE / MAX_BATCH_SIZE_120B
+ * (common/defines.h:30-31). */
+typedef struct {
+  int hidden;        /* H,  multiple of 64                     */
+  int inter;         /* IM, multiple of 64                     */
+  int experts;       /* E,  1..256                             */
+  int topk;          /* K,  must be 4 (EXPERT_PER_TOKEN)       */
+  int layers;        /* number of MoE layers held by the handle */
+  int max_tokens;    /* largest batch a forward call may carry */
+  float swiglu_limit;
+} moe_config;
+
+/* Stage indices for moe_profile_read. */
+enum {
+  MOE_STAGE_ROUTER = 0,   /* logits + bias + top-4 + softmax        */
+  MOE_STAGE_DISPATCH = 1, /* histogram + scan + stable permutation  */
+  MOE_STAGE_GATHER = 2,   /* rows copied into per-expert segments   */
+  MOE_STAGE_GATE_UP = 3,  /* grouped GEMM 1 + clamped SwiGLU        */
+  MOE_STAGE_DOWN = 4,     /* grouped GEMM 2 + bias                  */
+  MOE_STAGE_COMBINE = 5,  /* weighted sum back to token order       */
+  MOE_NUM_STAGES = 6
+};
+
+/* Allocates weights and workspaces for cfg on the current device.
+ * Replaces the allocation half of init_device_context_ep (expert.cpp:709-873)
+ * and init_device_context (getp_run.cpp:19-185). */
+int moe_create(const moe_config *cfg, moe_handle **out);
+
+/* Frees everything the handle owns.  Replaces cleanup_device_context_ep
+ * (expert.cpp:1234-1364). */
+int moe_destroy(moe_handle *h);
+
+/* Converts one layer's weights to bf16 (round to nearest even) and stores them
+ * in the device layout of the kernels.  Arguments are the reference's host
+ * pointers for that layer: w_router [E,H], b_router [E], w_mlp1 [E,2*IM,H]
+ * (rows alternate gate/up), b_mlp1 [E,2*IM], w_mlp2 [E,H,IM], b_mlp2 [E,H],
+ * all fp32 row-major (run.cpp:234-247).  Replaces the upload half of
+ * init_device_context_ep (expert.cpp:874-1009), getp_run.cpp:186-293 and
+ * pack_fp32_to_bf16_matmul (utility/utility.cpp:558-622).  Synchronous. */
+int moe_upload_layer(moe_handle *h, int layer, const float *w_router,
+                     const float *b_router, const float *w_mlp1,
+                     const float *b_mlp1, const float *w_mlp2,
+                     const float *b_mlp2);
+
+/* The whole layer for one batch: out[t,:] (+)= sum_k w[t,k] * expert_k(x[t,:]).
+ *   x    bf16 [n_tokens, H] row-major (the reference's d_t)
+ *   pos  int  [n_tokens] or NULL; pos[t] < 0 marks an inactive row, which takes
+ *        part in nothing (utility.cpp:281-282, :1071; matmul.cpp:955)
+ *   out  f32  [n_tokens, H] (the reference's d_e_agg).  accumulate != 0: the
+ *        result is added to out, as the reference does after zeroing it
+ *        (getp_run.cpp:719-720, utility.cpp:719-724); accumulate == 0: out is
+ *        overwritten and inactive rows are set to zero.
+ * Replaces getp_run.cpp:697-845 (router, top-k, local MoE path) and, with one
+ * GPU, gpu_forward_device_batch_ep (expert.cpp:1366-1607). */
+int moe_forward(moe_handle *h, int layer, const uint16_t *x, const int *pos,
+                int n_tokens, float *out, int accumulate, void *stream);
+
+/* Stage 1 alone.  Writes topk_i int [n_tokens,K] (descending score, ties to
+ * the lower expert id; -1 on inactive rows), topk_v f32 [n_tokens,K] (softmax
+ * over the K selected logits) and, if score != NULL, the logits f32
+ * [n_tokens,E].  Replaces matmul_router_kernel (matmul/matmul.cpp:945-1019)
+ * and fused_topk_softmax_batch_kernel (utility/utility.cpp:273-365), i.e. the
+ * producers of d_router_score, d_topk_i, d_topk_v (getp_run.cpp:697-716). */
+int moe_router(moe_handle *h, int layer, const uint16_t *x, const int *pos,
+               int n_tokens, float *score, int *topk_i, float *topk_v,
+               void *stream);
+
+/* Stage 2 alone, from caller-supplied routing.  Builds, inside the handle,
+ * offsets int [E+1] (exclusive scan of the per-expert histogram over active
+ * rows) and perm int [offsets[E]]: segment e lists the assignments t*K+k with
+ * topk_i[t,k] == e in increasing token order.  Replaces
+ * count_expert_assignments_kernel, exclusive_scan_small_kernel and
+ * build_expert_assignments_kernel (utility/utility.cpp:1058-1106, :758-777). */
+int moe_dispatch(moe_handle *h, const int *topk_i, const int *pos, int n_tokens,
+                 void *stream);
+
+/* Copies the result of the last dispatch to device buffers of the caller:
+ * offsets int [E+1], perm int [n_tokens*K] (entries past offsets[E] are -1).
+ * Either may be NULL. */
+int moe_get_dispatch(moe_handle *h, int *offsets, int *perm, int n_tokens,
+                     void *stream);
+
+/* Stages 2-6 from caller-supplied routing: the body of
+ * gpu_forward_device_batch_ep (expert.cpp:1366), which reads d_t, d_topk_i,
+ * d_topk_v, d_pos and adds into d_e_agg. */
+int moe_experts(moe_handle *h, int layer, const uint16_t *x, const int *pos,
+                const int *topk_i, const float *topk_v, int n_tokens,
+                float *out, int accumulate, void *stream);
+
+/* Per-stage timing with HIP events on the stream of the forward calls.
+ * moe_profile_enable(h, n) arms timing for the next n forward calls (n <= 256);
+ * moe_profile_read synchronises on the recorded events and returns the mean
+ * duration of every stage in milliseconds (ms[MOE_NUM_STAGES]) and the number
+ * of calls measured.  Replaces PROFILE_GPU_SCOPE (profiler/profiler.h:10-18). */
+int moe_profile_enable(moe_handle *h, int n_calls);
+int moe_profile_read(moe_handle *h, float *ms, int *n_calls);
+
+/* Sizes the kernels work with, for reports: number of row tiles the last
+ * dispatch produced is data dependent and stays on the device; these are the
+ * static figures. */
+size_t moe_weight_bytes(const moe_handle *h);    /* device bytes of one layer */
+size_t moe_workspace_bytes(const moe_handle *h); /* device bytes of workspaces */
+
+const char *moe_last_error(void);
+const char *moe_version(void);
+
+/* Device-memory helpers so that a host without a HIP toolchain (the ctypes test
+ * harness) can stage buffers.  Thin wrappers over hipMalloc / hipFree /
+ * hipMemcpy / hipMemset / hipDeviceSynchronize; not part of the reference. */
+int moe_dev_alloc(void **ptr, size_t bytes);
+int moe_dev_free(void *ptr);
+int moe_dev_upload(void *dst_dev, const void *src_host, size_t bytes);
+int moe_dev_download(void *dst_host, const void *src_dev, size_t bytes);
+int moe_dev_memset(void *dst_dev, int value, size_t bytes);
+int moe_dev_sync(void);
+int moe_dev_count(void);
+
+/* Wall-clock timing of back-to-back forward calls with HIP events on one
+ * stream: runs warmup untimed calls, then iters timed calls, and returns the
+ * total milliseconds of the timed calls.  Used by the benchmark. */
+int moe_time_forward(moe_handle *h, int layer, const uint16_t *x, const int *pos,
+                     int n_tokens, float *out, int warmup, int iters,
+                     float *total_ms);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MI355_MOE_ABI_H */
