@@ -1,0 +1,278 @@
+"""Parity of the HIP path (through the C-ABI) against the CPU oracle.
+
+Bars: expert ids, offsets and per-expert permutations bit-exact; layer outputs
+within max-abs 2e-2 and rel-L2 1e-3 of the oracle evaluated on the same
+bf16-representable inputs with the same rounding point (SwiGLU output to bf16).
+"""
+import numpy as np
+import pytest
+
+from gpt_oss_amd import abi, synth
+from oracle import binding as ob
+
+pytestmark = pytest.mark.gpu
+
+MAX_ABS = 2e-2
+REL_L2 = 1e-3
+W = ("w_router", "b_router", "w_mlp1", "b_mlp1", "w_mlp2", "b_mlp2")
+
+
+def rel_l2(a, b):
+    return float(np.linalg.norm(a.astype(np.float64) - b) / max(np.linalg.norm(b), 1e-30))
+
+
+def bf16_layer(shape, tokens=None, seed=0):
+    L = synth.make_layer(shape, seed=seed, tokens=tokens)
+    return {k: (synth.round_bf16(v) if v.dtype == np.float32 else v) for k, v in L.items()}
+
+
+def make_moe(shape, L, max_tokens):
+    m = abi.Moe(shape.hidden, shape.inter, shape.experts, max_tokens=max_tokens, swiglu_limit=shape.limit)
+    m.upload_layer(0, *[L[k] for k in W])
+    return m
+
+
+def oracle_rows(L, x, pos, rows, limit=7.0):
+    xs = np.ascontiguousarray(x[rows])
+    ps = None if pos is None else np.ascontiguousarray(pos[rows])
+    return ob.moe_layer(xs, ps, *[L[k] for k in W], 4, limit, mode=ob.ROUND_ACT_BF16 | ob.PAR_TOKENS)
+
+
+def check_routing(R, L, x, pos, E):
+    score, ti, tv = ob.router(x, pos, L["w_router"], L["b_router"], 4)
+    off, perm, _ = ob.dispatch(ti, pos, E)
+    assert np.array_equal(R["topk_i"], ti), "expert ids differ from the oracle"
+    act = np.ones(x.shape[0], bool) if pos is None else pos >= 0
+    np.testing.assert_allclose(R["score"][act], score[act], rtol=0, atol=2e-6)
+    np.testing.assert_allclose(R["topk_v"], tv, rtol=0, atol=1e-6)
+    assert np.array_equal(R["offsets"], off), "offsets differ"
+    assert np.array_equal(R["perm"][:off[-1]], perm), "per-expert permutation differs"
+    assert np.all(R["perm"][off[-1]:] == -1)
+    return ti, off
+
+
+def check_outputs(R, L, x, pos, rows, limit=7.0):
+    want = oracle_rows(L, x, pos, rows, limit)
+    got = R["out"][rows]
+    assert np.abs(got - want).max() <= MAX_ABS
+    assert rel_l2(got, want) <= REL_L2
+    return rel_l2(got, want)
+
+
+# ---------------- configuration 1 ----------------
+
+def test_c1_against_oracle_and_reference_vectors(golden, c1_layer):
+    sh = synth.CONFIGS["c1"]
+    L = {k: synth.round_bf16(c1_layer[k]) for k in W}
+    x = synth.round_bf16(golden["t"])
+    m = make_moe(sh, L, 64)
+    R = abi.run_layer(m, 0, x, None)
+    ti, _ = check_routing(R, L, x, None, sh.experts)
+    check_outputs(R, L, x, None, np.arange(64))
+    # Against the reference's fp32 forward() itself: the difference is the bf16
+    # quantisation of inputs, weights and activations (about 2^-9 relative per
+    # element), not kernel error, so the bound is looser and stated here: 1e-2.
+    same = np.all(np.sort(ti, axis=1) == np.sort(golden["topk_i"], axis=1), axis=1)
+    assert same.mean() >= 0.9
+    assert rel_l2(R["out"][same], golden["e_agg"][same]) <= 1e-2
+
+
+# ---------------- router ----------------
+
+@pytest.mark.parametrize("E,T", [(32, 4096), (128, 6144), (8, 50), (32, 1), (64, 333), (20, 100)])
+def test_router_bit_exact(E, T):
+    sh = synth.LayerShape("r", T, 2880, 64, E)
+    L = bf16_layer(sh)
+    pos = np.zeros(T, np.int32)
+    pos[5::11] = -1
+    m = make_moe(sh, L, T)
+    R = abi.run_layer(m, 0, L["x"], pos)
+    check_routing(R, L, L["x"], pos, E)
+    assert np.all(R["topk_i"][pos < 0] == -1) and np.all(R["topk_v"][pos < 0] == 0)
+    assert np.all(R["out"][pos < 0] == 0)
+
+
+def test_router_ties_go_to_lower_expert():
+    E, T, H = 32, 64, 256
+    sh = synth.LayerShape("ties", T, H, 64, E)
+    L = bf16_layer(sh)
+    wr = L["w_router"].copy()
+    br = L["b_router"].copy()
+    wr[8] = wr[16]; br[8] = br[16]          # equal logits on experts 8 and 16
+    wr[3] = wr[30] = wr[17]; br[3] = br[30] = br[17]
+    wr[20:24] = 0; br[20:24] = 0.5          # a four-way plateau
+    L["w_router"], L["b_router"] = wr, br
+    m = make_moe(sh, L, T)
+    R = abi.run_layer(m, 0, L["x"], None)
+    ti, _ = check_routing(R, L, L["x"], None, E)
+    both = np.isin(8, ti) if False else [(8 in r) and (16 in r) for r in ti]
+    for r in ti[np.array(both)]:
+        assert list(r).index(8) < list(r).index(16)
+    # all logits equal: the reference picks 0,1,2,3 (run.cpp:388-421 under a stable sort)
+    L["w_router"] = np.zeros_like(wr); L["b_router"] = np.zeros_like(br)
+    m2 = make_moe(sh, L, T)
+    R2 = abi.run_layer(m2, 0, L["x"], None)
+    assert np.all(R2["topk_i"] == np.arange(4, dtype=np.int32))
+    assert np.all(R2["topk_v"] == 0.25)
+
+
+# ---------------- dispatch ----------------
+
+def _dispatch_case(m, ti, pos, E):
+    T = ti.shape[0]
+    dti = abi.DevBuf.from_numpy(ti.astype(np.int32))
+    dpos = abi.DevBuf.from_numpy(pos.astype(np.int32)) if pos is not None else None
+    doff = abi.DevBuf((E + 1) * 4)
+    dperm = abi.DevBuf(max(T, 1) * 16)
+    m.dispatch(dti, dpos, T)
+    m.get_dispatch(doff, dperm, T)
+    abi.sync()
+    off = doff.download((E + 1,), np.int32)
+    perm = dperm.download((T * 4,), np.int32)
+    woff, wperm, _ = ob.dispatch(ti.astype(np.int32), pos, E)
+    assert np.array_equal(off, woff)
+    assert np.array_equal(perm[:woff[-1]], wperm)
+    assert np.all(perm[woff[-1]:] == -1)
+
+
+@pytest.mark.parametrize("E", [32, 128, 8])
+def test_dispatch_bit_exact(E):
+    rng = np.random.default_rng(E)
+    m = abi.Moe(64, 64, E, max_tokens=7168)
+    for T in (1, 63, 64, 257, 1000, 4096, 7168):
+        ti = np.stack([rng.permutation(E)[:4] for _ in range(T)]).astype(np.int32)
+        pos = np.where(rng.random(T) < 0.15, -1, 1).astype(np.int32)
+        _dispatch_case(m, ti, pos, E)
+        _dispatch_case(m, ti, None, E)
+    # heavy skew: every token picks experts 0..2 plus one of the rest; most experts empty
+    T = 3000
+    ti = np.tile(np.array([2, 0, 1, 0], np.int32), (T, 1))
+    ti[:, 3] = 3 + (np.arange(T) % 2) * (E - 4)
+    _dispatch_case(m, ti, None, E)
+    # nothing active
+    _dispatch_case(m, ti, np.full(T, -1, np.int32), E)
+
+
+# ---------------- whole layer at the benchmark shapes ----------------
+
+@pytest.fixture(scope="module")
+def c2():
+    sh = synth.CONFIGS["c2"]
+    L = bf16_layer(sh)
+    m = make_moe(sh, L, 7168)
+    return sh, L, m
+
+
+def test_c2_full_batch(c2):
+    sh, L, m = c2
+    T = sh.tokens
+    R = abi.run_layer(m, 0, L["x"], None)
+    _, off = check_routing(R, L, L["x"], None, sh.experts)
+    counts = np.diff(off)
+    assert counts.sum() == 4 * T and counts.min() > 300  # roughly uniform load
+    rows = np.random.default_rng(0).choice(T, 48, replace=False)
+    err = check_outputs(R, L, L["x"], None, np.sort(rows))
+    print(f"c2 rel-L2 vs oracle on 48 rows: {err:.2e}; rows per expert {counts.min()}..{counts.max()}")
+    assert np.isfinite(R["out"]).all()
+
+
+def test_c2_token_permutation_is_bit_exact(c2):
+    """A row's result does not depend on where the row sits in the batch."""
+    sh, L, m = c2
+    T = 1500
+    x = L["x"][:T]
+    p = np.random.default_rng(1).permutation(T)
+    a = abi.run_layer(m, 0, x, None)["out"]
+    b = abi.run_layer(m, 0, np.ascontiguousarray(x[p]), None)["out"]
+    assert np.array_equal(a[p], b)
+
+
+def test_c2_inactive_rows_equal_compaction(c2):
+    sh, L, m = c2
+    T = 900
+    x = L["x"][:T]
+    pos = np.where(np.random.default_rng(2).random(T) < 0.4, -1, 7).astype(np.int32)
+    a = abi.run_layer(m, 0, x, pos)["out"]
+    b = abi.run_layer(m, 0, np.ascontiguousarray(x[pos >= 0]), None)["out"]
+    assert np.array_equal(a[pos >= 0], b)
+    assert np.all(a[pos < 0] == 0)
+
+
+def test_c2_accumulate_and_caller_routing(c2):
+    sh, L, m = c2
+    T, H = 700, sh.hidden
+    x = L["x"][:T]
+    pos = np.zeros(T, np.int32)
+    pos[::9] = -1
+    base = abi.run_layer(m, 0, x, pos)
+    prior = np.random.default_rng(3).standard_normal((T, H)).astype(np.float32)
+    dx = abi.DevBuf.from_numpy(synth.to_bf16_bits(x))
+    dpos = abi.DevBuf.from_numpy(pos)
+    dout = abi.DevBuf.from_numpy(prior)
+    m.forward(0, dx, dpos, T, dout, accumulate=True)
+    abi.sync()
+    got = dout.download((T, H), np.float32)
+    assert np.array_equal(got[pos < 0], prior[pos < 0])
+    np.testing.assert_allclose(got[pos >= 0], prior[pos >= 0] + base["out"][pos >= 0], rtol=0, atol=1e-6)
+    # stages 2-6 from the caller's routing (the reference's gpu_forward_device_batch_ep contract)
+    dti = abi.DevBuf.from_numpy(base["topk_i"])
+    dtv = abi.DevBuf.from_numpy(base["topk_v"])
+    dout2 = abi.DevBuf(T * H * 4)
+    m.experts(0, dx, dpos, dti, dtv, T, dout2, accumulate=False)
+    abi.sync()
+    assert np.array_equal(dout2.download((T, H), np.float32), base["out"])
+
+
+@pytest.mark.parametrize("name", ["c3a", "c3b"])
+def test_c3_zipf_routing(name, c2):
+    sh = synth.CONFIGS[name]
+    _, L2, m = c2
+    L = dict(L2)
+    L["w_router"], L["b_router"] = [synth.round_bf16(a) for a in synth.make_router(sh)]
+    m.upload_layer(0, *[L[k] for k in W])
+    try:
+        x = synth.make_activations(sh)
+        R = abi.run_layer(m, 0, x, None)
+        _, off = check_routing(R, L, x, None, sh.experts)
+        counts = np.diff(off)
+        print(f"{name}: rows per expert max {counts.max()} min {counts.min()} (T={sh.tokens})")
+        assert counts.max() > 6 * max(counts.min(), 1)  # the load really is skewed
+        rows = np.sort(np.random.default_rng(4).choice(sh.tokens, 32, replace=False))
+        check_outputs(R, L, x, None, rows)
+    finally:
+        m.upload_layer(0, *[L2[k] for k in W])
+
+
+def test_c4_120b_shape():
+    sh = synth.CONFIGS["c4"]
+    L = bf16_layer(sh)
+    m = make_moe(sh, L, sh.tokens)
+    R = abi.run_layer(m, 0, L["x"], None)
+    check_routing(R, L, L["x"], None, sh.experts)
+    rows = np.sort(np.random.default_rng(5).choice(sh.tokens, 32, replace=False))
+    check_outputs(R, L, L["x"], None, rows)
+
+
+# ---------------- host logic on the GPU box ----------------
+
+def test_error_paths_and_profiling(c2):
+    sh, L, m = c2
+    dx = abi.DevBuf(16 * sh.hidden * 2)
+    dx.memset(0)
+    dout = abi.DevBuf(16 * sh.hidden * 4)
+    with pytest.raises(abi.MoeError) as e:
+        m.forward(0, dx, None, 7169, dout)
+    assert e.value.code == -3
+    with pytest.raises(abi.MoeError) as e:
+        m.forward(1, dx, None, 16, dout)
+    assert e.value.code == -1
+    fresh = abi.Moe(64, 64, 8, max_tokens=16)
+    with pytest.raises(abi.MoeError) as e:
+        fresh.forward(0, dx, None, 16, dout)
+    assert e.value.code == -5
+    m.forward(0, dx, None, 0, dout)  # empty batch is a no-op
+    m.profile_enable(3)
+    for _ in range(3):
+        m.forward(0, dx, None, 16, dout)
+    ms, n = m.profile_read()
+    assert n == 3 and all(v > 0 for v in ms.values())
