@@ -17,10 +17,6 @@ constexpr int kTileRows = 256;  // tallest row tile of the grouped GEMMs
 constexpr int kTileGran = 64;   // row tiles are multiples of this (2 wave rows x 32)
 constexpr float kAlpha = 1.702f;  // run.cpp:709
 
-// Column-tile widths in 32-column blocks per wave (2 wave columns per tile).
-constexpr int kNbwGateUp = 4;  // 256 columns: 64 gate/up pairs per wave
-constexpr int kNbwDown = 3;    // 192 columns
-
 // Per-expert record written by the scan kernel and read by the GEMMs.
 struct ExpertInfo {
   int row0;       // first padded row of the expert's segment (multiple of 64)

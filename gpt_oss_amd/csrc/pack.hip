@@ -26,7 +26,8 @@ __device__ __forceinline__ float bf16_round(float f) {
 // register layout of v_mfma_f32_32x32x16_bf16.  Fragments are ordered
 // [row block][k block].  With gate_up set, row block 2p holds the gate rows
 // (source rows 2j) and row block 2p+1 the up rows (source rows 2j+1) of
-// j = 32p .. 32p+31, so that a lane's gate and up accumulators line up.
+// j = 32p .. 32p+31, so that a lane's gate and up accumulators line up and the
+// SwiGLU epilogue needs no exchange between lanes.
 __global__ void pack_weight_kernel(const float *__restrict__ src, uint4 *__restrict__ dst, int rows,
                                    int cols, int gate_up) {
   const int kb_total = cols / kFragK;
