@@ -8,6 +8,7 @@ import sys
 PKG = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(PKG, "csrc")
 LIB = os.path.join(PKG, "libmi355_moe.so")
+PROBE = os.path.join(PKG, "ingest_probe.exe")
 SOURCES = ["moe_api.hip", "pack.hip", "router.hip", "dispatch.hip", "gemm.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
@@ -37,6 +38,13 @@ def build_lib(verbose: bool = True, extra: list[str] | None = None) -> str:
     if verbose:
         print(" ".join(cmd), flush=True)
     subprocess.check_call(cmd)
+    # stand-alone measurement tool (streaming ceilings, counter calibration)
+    cmd = [HIPCC, "--offload-arch=gfx950", "-O3", os.path.join(CSRC, "ingest_probe.hip"), "-o", PROBE]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError(f"hipcc failed on ingest_probe.hip:\n{r.stderr}")
     return LIB
 
 
