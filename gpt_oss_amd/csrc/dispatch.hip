@@ -57,8 +57,8 @@ __device__ __forceinline__ int block_exclusive_scan_256(int v, int *buf, int tid
 // Pass 2 (one workgroup): turns the per-workgroup counts into exclusive bases,
 // and builds per-expert offsets and the row-tile plan of the grouped GEMMs.
 // An expert with M rows gets n_mt = ceil(M / 256) tiles of equal height
-// 64 * rb, rb = ceil(M / (64 * n_mt)) in 1..4; its segment in the padded row
-// space is n_mt * 64 * rb rows long, so tiles never overlap the next expert.
+// 32 * rb, rb = ceil(M / (32 * n_mt)) in 1..8; its segment in the padded row
+// space is n_mt * 32 * rb rows long, so tiles never overlap the next expert.
 __global__ __launch_bounds__(256) void dispatch_scan_kernel(int *__restrict__ blk_counts, int n_blk,
                                                            int E, int *__restrict__ offsets,
                                                            ExpertInfo *__restrict__ info,

@@ -6,25 +6,39 @@
 //
 // Data layout.  Both operands arrive as ready-made MFMA fragments of 1 KB
 // (64 lanes x 8 bf16, see pack.hip and gather_rows_kernel), ordered
-// [row block of 32][k block of 16], so every global load is a contiguous
-// 16 bytes per lane and lands in LDS in register order: LDS reads are
-// lane-linear ds_read_b128, free of bank conflicts by construction.
+// [row block of 32][k block of 16]: every global load is a contiguous 16
+// bytes per lane and is already in register order.
 //
-// Tiling.  A workgroup of WM x WN waves owns a tile of (WM*RB*32) rows x
-// (WN*NBW*32) columns of one expert; a wave keeps RB x NBW accumulators of
-// 32x32.  RB follows the expert's row count (ExpertInfo::rb) so that ragged
-// segments pad to at most 63 rows.  The reduction runs in steps of KPS k
-// blocks through a 4-stage LDS ring that global_load_lds (DMA into LDS, no
-// staging registers) keeps three steps ahead of the MFMAs.
+// Tiling.  A workgroup of NW waves owns a tile of (RBT*32) rows x
+// (NW*NBW*32) columns of one expert.  The waves split the columns only: each
+// wave keeps RBT x NBW accumulators of 32x32 over all rows of the tile, RBT =
+// 1..8 following the expert's row count (ExpertInfo::rb), so ragged segments
+// pad to at most 31 rows per tile and MFMA work follows the real rows.
+//
+// Feeding the matrix cores.  What bounds this kernel is how fast one CU can
+// take data in from L2 (about 45 GB/s with 100 KB in flight, 55-60 GB/s with
+// 200 KB), so the design maximises bytes in flight:
+//   * the row operand (shared by all waves) goes straight into an R-stage LDS
+//     ring by DMA (global_load_lds_dwordx4), R-1 steps ahead of the MFMAs;
+//   * the column operand is private to a wave in this layout, so it never
+//     touches LDS: it is loaded into an R-slot ring of VGPRs, R-1 steps ahead.
+// With R = 7 that is 6 steps x 32 KB = 192 KB in flight per CU.  Loads return
+// in order, so waiting for "all but the newest n" (s_waitcnt vmcnt(n)) picks out
+// exactly the step that is needed next and leaves the later ones in flight.
 //
 // Tile order.  Workgroup ids are dealt round-robin to the 8 XCDs, each with
 // its own L2.  Logical tile ids are laid out (expert, column tile, row tile)
 // with the row tile fastest, and XCD x takes the x-th contiguous eighth of
 // them: the tiles an XCD runs at one time share the expert's rows and a few
 // column slabs of its weights, so each weight byte leaves HBM once.
+#include <type_traits>
+
 #include "moe_internal.h"
 
 namespace moe {
+
+template <int V>
+using IC = std::integral_constant<int, V>;
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
@@ -43,9 +57,7 @@ __device__ __forceinline__ float swiglu(float g, float u, float limit) {
   return g * s * (u + 1.0f);
 }
 
-// s_waitcnt with only the vector-memory counter constrained (gfx9 encoding).
-#define WAIT_VMCNT(n) \
-  __builtin_amdgcn_s_waitcnt(((n) & 0xf) | (((n) >> 4) << 14) | (0x7 << 4) | (0xf << 8))
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 struct TileCoord {
   int e;      // expert
@@ -82,215 +94,260 @@ __device__ __forceinline__ bool locate_tile(const ExpertInfo *__restrict__ info,
   tc.e = e;
   tc.nt = rem / inf.n_mt;
   rb = inf.rb;
-  tc.rows0 = mt * 2 * rb * kRowBlock;
+  tc.rows0 = mt * rb * kRowBlock;
   tc.rb0 = (inf.row0 + tc.rows0) / kRowBlock;
   return true;
 }
 
-// LDS ring: one __shared__ array per stage, so that the compiler can tell a
-// read of one stage from the DMA that fills another and does not serialise them.
-template <int NST>
-struct StageRing {
-  uint4 *p[NST];
-};
+// ---- vector-memory instructions of the main loop ----
+
+// 16 bytes per lane from global memory straight into LDS at base + 16*lane
+// (global_load_lds_dwordx4; the LDS base must be wave-uniform).
+__device__ __forceinline__ void dma_to_lds_16(const uint4 *g, uint4 *lds_wave_base) {
+  __builtin_amdgcn_global_load_lds(g, lds_wave_base, 16, 0, 0);
+}
+
+// s_waitcnt with only the vector-memory counter constrained (gfx9 encoding).
+// Loads return in order, so "at most n outstanding" means "all but the newest n
+// have landed".  The compiler places its own waits before the first use of
+// loaded data in the same wave; these explicit ones stand before the barriers,
+// where other waves are about to read what this wave's DMA wrote.
+#define WAIT_VMCNT(n) \
+  __builtin_amdgcn_s_waitcnt(((n) & 0xf) | (((n) >> 4) << 14) | (0x7 << 4) | (0xf << 8))
 
 // Workgroup barrier that orders LDS traffic only.  A __syncthreads (or a
 // workgroup fence) would also drain the vector-memory counter and with it the
-// DMA of the steps still in flight; those are covered by the explicit vmcnt
-// waits of the pipeline.  The memory clobber keeps the compiler from moving
-// LDS accesses across the barrier.
+// loads of the steps still in flight.  The memory clobber keeps the compiler
+// from moving memory accesses across the barrier.
 __device__ __forceinline__ void lds_barrier() {
   asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 }
 
-// 16 bytes per lane from global memory straight into LDS at base + 16*lane
-// (global_load_lds_dwordx4; M0 carries the wave-uniform LDS base).  Issued as
-// inline assembly on purpose: the compiler then does not pair the LDS write with
-// later ds_reads of OTHER stages and drain the whole queue before them; the
-// pipeline's own vmcnt waits order the read of a stage after its fill.
-__device__ __forceinline__ void dma_to_lds_16(const uint4 *g, uint4 *lds_wave_base) {
-  const uint32_t m = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint4 *)lds_wave_base;
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
-               :
-               : "s"(m), "v"(g)
-               : "memory");
-}
-
-// Shape of one workgroup: WM x WN waves, each owning RB x NBW accumulators of
-// 32x32; the tile is (WM*RB*32) rows x (WN*NBW*32) columns.  KPS k blocks per
-// pipeline step, NST LDS stages.
-template <int WM_, int WN_, int NBW_, int KPS_, int NST_>
-struct GemmCfg {
-  static constexpr int WM = WM_, WN = WN_, NBW = NBW_, KPS = KPS_, NST = NST_;
-  static constexpr int NW = WM * WN;              // waves
-  static constexpr int THREADS = NW * 64;
-  static constexpr int RB_MAX = kTileRows / (WM * kRowBlock);
-  static constexpr int TILE_NB = WN * NBW;        // column blocks per tile
-  static constexpr int B_OFF = WM * RB_MAX * KPS * 64;             // B follows the tallest A, in uint4
-  static constexpr int STAGE = (WM * RB_MAX + WN * NBW) * KPS * 64;  // uint4 per stage
+template <int R>
+struct StageRing {
+  uint4 *p[R];
 };
 
-template <int RB, typename C, bool GATE_UP>
+// NW waves side by side over the columns, NBW column blocks per wave, R ring
+// slots (LDS stages for the row operand, register slots for the column operand).
+template <int NW_, int NBW_, int R_>
+struct GemmCfg {
+  static constexpr int NW = NW_, NBW = NBW_, R = R_, KPS = 2;
+  static constexpr int THREADS = NW * 64;
+  static constexpr int TILE_NB = NW * NBW;              // column blocks per tile
+  static constexpr int RBT_MAX = kTileRows / kRowBlock;  // row blocks per tile, at most
+  static constexpr int STAGE = RBT_MAX * KPS * 64;       // uint4 per LDS stage (16 KB)
+};
+
+template <int RBT, typename C, bool GATE_UP>
 __device__ __forceinline__ void gemm_tile(const uint4 *__restrict__ a_frag,  // [rb][KB][64]
                                           const uint4 *__restrict__ b_frag,  // expert: [nb][KB][64]
                                           int KB, int rb0, int nb0, int nb_valid,
                                           const float *__restrict__ bias_a,  // gate / down bias (expert)
                                           const float *__restrict__ bias_b,  // up bias (expert)
                                           void *__restrict__ outp, int out_ld, float limit,
-                                          const StageRing<C::NST> &ring) {
-  constexpr int WN = C::WN, NBW = C::NBW, KPS = C::KPS, NST = C::NST, NW = C::NW;
+                                          // One __restrict__ pointer per LDS stage: after
+                                          // inlining the compiler can tell a read of one stage
+                                          // from the DMA that fills another and waits only for
+                                          // the fill of the stage it reads.
+                                          uint4 *__restrict__ s0, uint4 *__restrict__ s1,
+                                          uint4 *__restrict__ s2, uint4 *__restrict__ s3,
+                                          uint4 *__restrict__ s4, uint4 *__restrict__ s5,
+                                          uint4 *__restrict__ s6) {
+  StageRing<C::R> ring;
+  ring.p[0] = s0; ring.p[1] = s1; ring.p[2] = s2; ring.p[3] = s3;
+  ring.p[4] = s4; ring.p[5] = s5; ring.p[6] = s6;
+  constexpr int NBW = C::NBW, KPS = C::KPS, R = C::R, NW = C::NW;
   static_assert(KPS == 2, "the step is software-pipelined as two k blocks");
-  constexpr int A_CH = C::WM * RB * KPS;  // 1 KB chunks of A per stage
-  constexpr int B_CH = WN * NBW * KPS;    // 1 KB chunks of B per stage
-  static_assert(A_CH % NW == 0 && B_CH % NW == 0, "every wave issues the same number of loads");
-  constexpr int LPS = (A_CH + B_CH) / NW;  // DMA loads per wave per step
-  constexpr int NF = RB + NBW;             // fragments a wave reads per k block
-  constexpr int NM = RB * NBW;             // MFMAs per k block
-  constexpr int SIDE1 = (NF + NM - 1) / NM;        // side items per MFMA, first k block
-  constexpr int SIDE2 = (LPS + NF + NM - 1) / NM;  // second k block
+  constexpr int A_CH = RBT * KPS;            // 1 KB chunks of the row operand per step
+  constexpr int LA = (A_CH + NW - 1) / NW;   // DMA loads per wave per step (a short last pass repeats a chunk)
+  constexpr int LB = NBW * KPS;              // register loads per wave per step
+  constexpr int LPS = LA + LB;
+  static_assert(LPS * (R - 2) + LA <= 63, "vmcnt is a 6-bit counter");
+  constexpr int NM = RBT * NBW;              // MFMAs per k block
+  constexpr int SIDE = (RBT + LB + NM - 1) / NM;  // side items per MFMA
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int wm = w / WN, wn = w % WN;
 
-  f32x16 acc[RB][NBW];
+  f32x16 acc[RBT][NBW];
 #pragma unroll
-  for (int i = 0; i < RB; i++)
+  for (int i = 0; i < RBT; i++)
 #pragma unroll
     for (int j = 0; j < NBW; j++)
 #pragma unroll
       for (int q = 0; q < 16; q++) acc[i][j][q] = 0.f;
 
-  // DMA chunk c of a stage (c = pass*NW + wave) covers row block c / KPS, k block
-  // c % KPS.  Load m (0 <= m < LPS) of this wave: first its A chunks, then its B chunks.
   const uint4 *a_src = a_frag + (size_t)rb0 * KB * 64 + lane;
-  const uint4 *b_src = b_frag + (size_t)nb0 * KB * 64 + lane;
-  auto issue_one = [&](uint4 *st, int ks, int m) {
-    if (m < A_CH / NW) {
-      const int c = m * NW + w;
-      const uint4 *g = a_src + ((size_t)(c / KPS) * KB + ks * KPS + c % KPS) * 64;
-      dma_to_lds_16(g, st + c * 64);
-    } else {
-      const int c = (m - A_CH / NW) * NW + w;
-      // Column blocks past the end of the matrix (last column tile only) re-load
-      // the last valid block instead of branching; their products are never stored.
-      const int nb = min(c / KPS, nb_valid - 1);
-      const uint4 *g = b_src + ((size_t)nb * KB + ks * KPS + c % KPS) * 64;
-      dma_to_lds_16(g, st + C::B_OFF + c * 64);
-    }
-  };
-  auto issue = [&](uint4 *st, int ks) {
+  // Column blocks past the end of the matrix (last column tile only) re-load
+  // the last valid block; their products are never stored.
+  const uint4 *b_src[NBW];
 #pragma unroll
-    for (int m = 0; m < LPS; m++) issue_one(st, ks, m);
-  };
+  for (int j = 0; j < NBW; j++)
+    b_src[j] = b_frag + (size_t)(nb0 + min(w * NBW + j, nb_valid - 1)) * KB * 64 + lane;
 
-  // Two register sets of fragments: while the MFMAs of one k block run, the
+  // Row operand: chunk c of a step (c = pass*NW + wave) is row block c / KPS, k block c % KPS.
+  auto issue_a = [&](uint4 *st, int ks, int m) {
+    const int c = min(m * NW + w, A_CH - 1);
+    dma_to_lds_16(a_src + ((size_t)(c / KPS) * KB + ks * KPS + c % KPS) * 64, st + c * 64);
+  };
+  // Column operand: register m of a slot is column block m / KPS, k block m % KPS.
+  u32x4 bq[R][LB];
+  auto issue_b = [&](int slot, int ks, int m) {
+    bq[slot][m] = *reinterpret_cast<const u32x4 *>(b_src[m / KPS] + (size_t)(ks * KPS + m % KPS) * 64);
+  };
+  // Two register sets of row fragments: while the MFMAs of one k block run, the
   // fragments of the next are read from LDS.
-  bf16x8 fa[2][RB], fb[2][NBW];
-  auto read_frag = [&](const uint4 *st, int kk, int buf, int f) {
-    if (f < RB) {
-      fa[buf][f] = __builtin_bit_cast(bf16x8, st[((wm * RB + f) * KPS + kk) * 64 + lane]);
-    } else {
-      fb[buf][f - RB] =
-          __builtin_bit_cast(bf16x8, st[C::B_OFF + ((wn * NBW + f - RB) * KPS + kk) * 64 + lane]);
-    }
+  bf16x8 fa[2][RBT];
+  auto read_a = [&](const uint4 *st, int kk, int buf, int i) {
+    fa[buf][i] = __builtin_bit_cast(bf16x8, st[(i * KPS + kk) * 64 + lane]);
   };
+  // "all but the newest k steps have landed", k = 0 .. R-2
+#define MOE_WAIT_STEPS(k)                            \
+  switch (k) {                                       \
+    case 0: WAIT_VMCNT(0); break;                    \
+    case 1: WAIT_VMCNT(LPS * (R > 2 ? 1 : 0)); break; \
+    case 2: WAIT_VMCNT(LPS * (R > 3 ? 2 : 0)); break; \
+    case 3: WAIT_VMCNT(LPS * (R > 4 ? 3 : 0)); break; \
+    case 4: WAIT_VMCNT(LPS * (R > 5 ? 4 : 0)); break; \
+    default: WAIT_VMCNT(LPS * (R > 6 ? 5 : 0)); break; \
+  }
+  static_assert(R == 7, "the step sequence below is written out for 7 slots");
 
+  // Issue order per wave: A(0) B(0) A(1) B(1) ... ; at the top of step ks the row
+  // operand is issued through step ks+R-1 and the column operand through ks+R-2.
   const int n_steps = KB / KPS;
 #pragma unroll
-  for (int s = 0; s < NST - 1; s++)
-    if (s < n_steps) issue(ring.p[s], s);
-  if (n_steps - 1 >= NST - 2) {
-    WAIT_VMCNT(LPS * (NST - 2));
+  for (int s = 0; s < R - 1; s++) {
+    if (s < n_steps) {
+#pragma unroll
+      for (int m = 0; m < LA; m++) issue_a(ring.p[s], s, m);
+#pragma unroll
+      for (int m = 0; m < LB; m++) issue_b(s, s, m);
+    }
+  }
+  if (R - 1 < n_steps) {
+#pragma unroll
+    for (int m = 0; m < LA; m++) issue_a(ring.p[R - 1], R - 1, m);
+    WAIT_VMCNT(LPS * (R - 2) + LA);
   } else {
     WAIT_VMCNT(0);
   }
   lds_barrier();
-  if (NST - 1 < n_steps) issue(ring.p[NST - 1], NST - 1);
 #pragma unroll
-  for (int f = 0; f < NF; f++) read_frag(ring.p[0], 0, 0, f);
+  for (int i = 0; i < RBT; i++) read_a(ring.p[0], 0, 0, i);
 
-  // Step ks: [read k block 1 | MFMAs of k block 0] [wait for step ks+1, barrier]
-  // [refill the stage just drained with step ks+NST, read k block 0 of step ks+1 |
-  // MFMAs of k block 1].  The side work is spread one item per MFMA so that it
-  // issues in the shadow of the matrix pipe.
-  for (int ks0 = 0; ks0 < n_steps; ks0 += NST) {
+  // Step ks, slot u = ks % R:
+  //   [MFMAs of k block 0 | read row fragments of k block 1, load B(ks+R-1) into slot u-1]
+  //   wait until step ks+1 has arrived, barrier
+  //   [MFMAs of k block 1 | DMA A(ks+R) into stage u, read row fragments of step ks+1]
+  // The side work is spread over the MFMAs so that it issues in their shadow.
+  // STEADY steps (every refill exists) carry no branch at all, so the whole
+  // group of R steps is one straight block; the last steps of the tile run the
+  // same code with the refills guarded.
+  auto step = [&](auto u_c, auto steady_c, int ks) {
+    constexpr int u = decltype(u_c)::value;
+    constexpr bool STEADY = decltype(steady_c)::value;
+    const uint4 *cur = ring.p[u];
+    const bool refill_b = STEADY || ks + R - 1 < n_steps;
 #pragma unroll
-    for (int u = 0; u < NST; u++) {
-      const int ks = ks0 + u;
-      if (ks < n_steps) {
-      const uint4 *cur = ring.p[u];
+    for (int m = 0; m < NM; m++) {
 #pragma unroll
-      for (int m = 0; m < NM; m++) {
-#pragma unroll
-        for (int t = m * SIDE1; t < (m + 1) * SIDE1; t++)
-          if (t < NF) read_frag(cur, 1, 1, t);
-        acc[m / NBW][m % NBW] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-            fa[0][m / NBW], fb[0][m % NBW], acc[m / NBW][m % NBW], 0, 0, 0);
-        __builtin_amdgcn_sched_barrier(0);
-      }
-      const bool more = ks + 1 < n_steps;
-      const bool refill = ks + NST < n_steps;
-      if (more) {
-        if (ks + NST - 1 < n_steps) {
-          WAIT_VMCNT(LPS * (NST - 2));  // all but the NST-2 newest steps have landed
-        } else {
-          WAIT_VMCNT(0);
+      for (int t = m * SIDE; t < (m + 1) * SIDE; t++) {
+        if (t < RBT) {
+          read_a(cur, 1, 1, t);
+        } else if (t < RBT + LB) {
+          if (refill_b) issue_b((u + R - 1) % R, ks + R - 1, t - RBT);
         }
-        lds_barrier();  // step ks+1 is complete in LDS; every wave is done with stage u
       }
-      const uint4 *nxt = ring.p[(u + 1) % NST];
-#pragma unroll
-      for (int m = 0; m < NM; m++) {
-#pragma unroll
-        for (int t = m * SIDE2; t < (m + 1) * SIDE2; t++) {
-          if (t < LPS) {
-            if (refill) issue_one(ring.p[u], ks + NST, t);
-          } else if (t < LPS + NF) {
-            if (more) read_frag(nxt, 0, 0, t - LPS);
-          }
-        }
-        acc[m / NBW][m % NBW] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-            fa[1][m / NBW], fb[1][m % NBW], acc[m / NBW][m % NBW], 0, 0, 0);
-        __builtin_amdgcn_sched_barrier(0);
-      }
-      }
+      acc[m / NBW][m % NBW] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+          fa[0][m / NBW], __builtin_bit_cast(bf16x8, bq[u][(m % NBW) * KPS + 0]),
+          acc[m / NBW][m % NBW], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
     }
+    const bool more = STEADY || ks + 1 < n_steps;
+    if (more) {
+      // loads issued after B(ks+1): steps ks+2 .. min(ks+R-1, n_steps-1)
+      if (STEADY) {
+        WAIT_VMCNT(LPS * (R - 2));
+      } else {
+        MOE_WAIT_STEPS(min(R - 2, n_steps - 2 - ks))
+      }
+      lds_barrier();  // step ks+1 is complete in LDS; every wave is done with stage u
+    }
+    const bool refill_a = STEADY || ks + R < n_steps;
+    const uint4 *nxt = ring.p[(u + 1) % R];
+#pragma unroll
+    for (int m = 0; m < NM; m++) {
+#pragma unroll
+      for (int t = m * SIDE; t < (m + 1) * SIDE; t++) {
+        if (t < LA) {
+          if (refill_a) issue_a(ring.p[u], ks + R, t);
+        } else if (t < LA + RBT) {
+          if (more) read_a(nxt, 0, 0, t - LA);
+        }
+      }
+      acc[m / NBW][m % NBW] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+          fa[1][m / NBW], __builtin_bit_cast(bf16x8, bq[u][(m % NBW) * KPS + 1]),
+          acc[m / NBW][m % NBW], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+  int ks0 = 0;
+  for (; ks0 + 2 * R - 2 < n_steps; ks0 += R) {
+    step(IC<0>{}, std::true_type{}, ks0 + 0);
+    step(IC<1>{}, std::true_type{}, ks0 + 1);
+    step(IC<2>{}, std::true_type{}, ks0 + 2);
+    step(IC<3>{}, std::true_type{}, ks0 + 3);
+    step(IC<4>{}, std::true_type{}, ks0 + 4);
+    step(IC<5>{}, std::true_type{}, ks0 + 5);
+    step(IC<6>{}, std::true_type{}, ks0 + 6);
   }
+  for (; ks0 < n_steps; ks0 += R) {
+    if (ks0 + 0 < n_steps) step(IC<0>{}, std::false_type{}, ks0 + 0);
+    if (ks0 + 1 < n_steps) step(IC<1>{}, std::false_type{}, ks0 + 1);
+    if (ks0 + 2 < n_steps) step(IC<2>{}, std::false_type{}, ks0 + 2);
+    if (ks0 + 3 < n_steps) step(IC<3>{}, std::false_type{}, ks0 + 3);
+    if (ks0 + 4 < n_steps) step(IC<4>{}, std::false_type{}, ks0 + 4);
+    if (ks0 + 5 < n_steps) step(IC<5>{}, std::false_type{}, ks0 + 5);
+    if (ks0 + 6 < n_steps) step(IC<6>{}, std::false_type{}, ks0 + 6);
+  }
+#undef MOE_WAIT_STEPS
 
   // Epilogue.  Accumulator register q of lane l is row 8*(q/4) + 4*(l/32) + q%4,
   // column l % 32 of its 32x32 block.  Results are re-ordered through LDS (the
-  // pipeline stages are idle now; each wave takes a private piece) so that they
-  // leave as 16 bytes per lane, 1 KB contiguous per wave store.
+  // ring is idle now; each wave takes a stage of its own) so that they leave as
+  // 16 bytes per lane, 1 KB contiguous per wave store.
   lds_barrier();  // every wave has finished reading the stages
-  static_assert(NW <= NST, "one stage per wave serves as its epilogue buffer");
+  static_assert(NW <= R, "one stage per wave serves as its epilogue buffer");
   uint4 *ebuf = ring.p[w];
   const int n = lane & 31;
   const int rsub = 4 * (lane >> 5);
+  if (w * NBW >= nb_valid) return;  // a wave without columns (last column tile only)
   if (GATE_UP) {
     // Column blocks come in (gate, up) pairs (see pack_weight_kernel): blocks 2P
     // and 2P+1 of the product hold gate_j and up_j of j = 32P .. 32P+31 in the
     // same lane and register.  The activation goes out as bf16 in the fragment
-    // order the down GEMM reads as its A operand: column j is k block j/16,
+    // order the down GEMM reads as its row operand: column j is k block j/16,
     // lane ((j%16)/8)*32 + row, element j % 8.
     static_assert(NBW % 2 == 0, "gate and up blocks of a pair must sit in one wave");
     static_assert(NBW * 64 <= C::STAGE, "epilogue buffer");
     uint4 *act = reinterpret_cast<uint4 *>(outp);
     uint16_t *e16 = reinterpret_cast<uint16_t *>(ebuf);
     const int kb2_total = out_ld / kFragK;
-    const int P0 = (nb0 + wn * NBW) >> 1;       // first pair of this wave
-    const int pairs_valid = (nb_valid - wn * NBW) >> 1;  // may be <= 0 in the last column tile
+    const int P0 = (nb0 + w * NBW) >> 1;              // first pair of this wave
+    const int pairs_valid = (nb_valid - w * NBW) >> 1;  // >= 1 here
     float bg[NBW / 2], bu[NBW / 2];
 #pragma unroll
     for (int p = 0; p < NBW / 2; p++) {
-      const int P = min(P0 + p, ((nb0 + nb_valid) >> 1) - 1);
+      const int P = P0 + min(p, pairs_valid - 1);
       bg[p] = bias_a[kRowBlock * P + n];
       bu[p] = bias_b[kRowBlock * P + n];
     }
     // element offset of (row 0, column n of pair p) inside the wave's buffer of NBW fragments
     const int e_off = ((n >> 4) * 64 + ((n & 15) >> 3) * 32) * 8 + (n & 7);
 #pragma unroll
-    for (int i = 0; i < RB; i++) {
+    for (int i = 0; i < RBT; i++) {
 #pragma unroll
       for (int p = 0; p < NBW / 2; p++) {
         uint16_t *dst = e16 + p * 2 * 64 * 8 + e_off;
@@ -301,7 +358,7 @@ __device__ __forceinline__ void gemm_tile(const uint4 *__restrict__ a_frag,  // 
               swiglu(acc[i][2 * p][q] + bg[p], acc[i][2 * p + 1][q] + bu[p], limit));
         }
       }
-      uint4 *row_dst = act + ((size_t)(rb0 + wm * RB + i) * kb2_total + 2 * P0) * 64 + lane;
+      uint4 *row_dst = act + ((size_t)(rb0 + i) * kb2_total + 2 * P0) * 64 + lane;
 #pragma unroll
       for (int f = 0; f < NBW; f++) {
         const uint4 v = ebuf[f * 64 + lane];
@@ -315,13 +372,11 @@ __device__ __forceinline__ void gemm_tile(const uint4 *__restrict__ a_frag,  // 
     float *ef = reinterpret_cast<float *>(ebuf);
     float bb[NBW];
 #pragma unroll
-    for (int j = 0; j < NBW; j++) {
-      const int b = min(nb0 + wn * NBW + j, nb0 + nb_valid - 1);
-      bb[j] = bias_a[kRowBlock * b + n];
-    }
-    const int col0 = kRowBlock * (nb0 + wn * NBW);
+    for (int j = 0; j < NBW; j++)
+      bb[j] = bias_a[kRowBlock * (nb0 + min(w * NBW + j, nb_valid - 1)) + n];
+    const int col0 = kRowBlock * (nb0 + w * NBW);
 #pragma unroll
-    for (int i = 0; i < RB; i++) {
+    for (int i = 0; i < RBT; i++) {
 #pragma unroll
       for (int j = 0; j < NBW; j++)
 #pragma unroll
@@ -329,14 +384,14 @@ __device__ __forceinline__ void gemm_tile(const uint4 *__restrict__ a_frag,  // 
           const int r = 8 * (q >> 2) + rsub + (q & 3);
           ef[r * LD + 32 * j + n] = acc[i][j][q] + bb[j];
         }
-      const size_t row0 = (size_t)(rb0 + wm * RB + i) * kRowBlock;
+      const size_t row0 = (size_t)(rb0 + i) * kRowBlock;
 #pragma unroll
       for (int t = 0; t < NBW * 4; t++) {
         const int idx = t * 64 + lane;
         const int r = idx / (NBW * 8);
         const int c4 = idx % (NBW * 8);
         const float4 v = *reinterpret_cast<const float4 *>(ef + r * LD + 4 * c4);
-        if (wn * NBW + c4 / 8 < nb_valid)
+        if (w * NBW + c4 / 8 < nb_valid)
           *reinterpret_cast<float4 *>(y + (row0 + r) * out_ld + col0 + 4 * c4) = v;
       }
     }
@@ -349,16 +404,10 @@ __global__ __launch_bounds__(C::THREADS) void grouped_gemm_kernel(
     const float *__restrict__ bias_a, const float *__restrict__ bias_b,
     const ExpertInfo *__restrict__ info, const int *__restrict__ totals, void *__restrict__ outp,
     int K, int N, int E, float limit) {
-  constexpr int NST = C::NST;
-  __shared__ uint4 st0[C::STAGE];
-  __shared__ uint4 st1[C::STAGE];
-  __shared__ uint4 st2[NST > 2 ? C::STAGE : 1];
-  __shared__ uint4 st3[NST > 3 ? C::STAGE : 1];
-  StageRing<NST> ring;
-  ring.p[0] = st0;
-  ring.p[1] = st1;
-  if constexpr (NST > 2) ring.p[2] = st2;
-  if constexpr (NST > 3) ring.p[3] = st3;
+  constexpr int R = C::R;
+  static_assert(R == 7, "seven stage arrays are declared below");
+  __shared__ uint4 st0[C::STAGE], st1[C::STAGE], st2[C::STAGE], st3[C::STAGE], st4[C::STAGE],
+      st5[C::STAGE], st6[C::STAGE];
   const int KB = K / kFragK;
   const int nb_total = (GATE_UP ? 2 * N : N) / kRowBlock;  // weight row blocks per expert
   const int n_ct = (nb_total + C::TILE_NB - 1) / C::TILE_NB;
@@ -370,24 +419,20 @@ __global__ __launch_bounds__(C::THREADS) void grouped_gemm_kernel(
   const uint4 *b_frag = w_frag + (size_t)tc.e * nb_total * KB * 64;
   const float *ba = bias_a + (size_t)tc.e * N;
   const float *bb = GATE_UP ? bias_b + (size_t)tc.e * N : nullptr;
+#define MOE_TILE_CASE(n) \
+  case n: gemm_tile<n, C, GATE_UP>(a_frag, b_frag, KB, tc.rb0, nb0, nb_valid, ba, bb, outp, N, limit, st0, st1, st2, st3, st4, st5, st6); break;
   switch (rb) {
-    case 1: gemm_tile<1, C, GATE_UP>(a_frag, b_frag, KB, tc.rb0, nb0, nb_valid, ba, bb, outp, N, limit, ring); break;
-    case 2: gemm_tile<2, C, GATE_UP>(a_frag, b_frag, KB, tc.rb0, nb0, nb_valid, ba, bb, outp, N, limit, ring); break;
-    case 3: gemm_tile<3, C, GATE_UP>(a_frag, b_frag, KB, tc.rb0, nb0, nb_valid, ba, bb, outp, N, limit, ring); break;
-    default: gemm_tile<4, C, GATE_UP>(a_frag, b_frag, KB, tc.rb0, nb0, nb_valid, ba, bb, outp, N, limit, ring); break;
+    MOE_TILE_CASE(1) MOE_TILE_CASE(2) MOE_TILE_CASE(3) MOE_TILE_CASE(4)
+    MOE_TILE_CASE(5) MOE_TILE_CASE(6) MOE_TILE_CASE(7)
+    default: gemm_tile<8, C, GATE_UP>(a_frag, b_frag, KB, tc.rb0, nb0, nb_valid, ba, bb, outp, N, limit, st0, st1, st2, st3, st4, st5, st6); break;
   }
+#undef MOE_TILE_CASE
 }
 
-// 4 waves (2 x 2), one per SIMD, each with 4 x 5 accumulators (320 registers).
-// Tiles are 256 x 320: a CU takes in at most about 21 bytes per clock from L2,
-// so the arithmetic per byte of the tile, 2*256*320 flops per (256+320)*2
-// bytes for every unit of k, bounds the MFMA rate; 320 also divides both
-// 2*IM = 5760 and H = 2880 at the GPT-OSS shapes, so no column tile is partial.
-// 2 k blocks per step, 4 stages of 36 KB.
-using CfgGateUp = GemmCfg<2, 2, 4, 2, 4>;
-using CfgDown = GemmCfg<2, 2, 4, 2, 4>;
-static_assert(CfgGateUp::WM == 2 && CfgDown::WM == 2,
-              "ExpertInfo::rb counts fragments per wave row for two wave rows (kTileGran = 64)");
+// 4 waves, one per SIMD, each 256 rows x 64 columns (8 x 2 accumulators = all
+// 256 accumulation registers); 256 x 256 tiles; 7 ring slots.
+using CfgGemm = GemmCfg<4, 2, 7>;
+static_assert(CfgGemm::RBT_MAX * kRowBlock == kTileRows, "tile plan of dispatch_scan_kernel");
 
 template <typename C, bool GATE_UP>
 static hipError_t launch_gemm(const uint4 *a, const uint4 *w, const float *ba, const float *bb,
@@ -404,15 +449,15 @@ static hipError_t launch_gemm(const uint4 *a, const uint4 *w, const float *ba, c
 hipError_t launch_gate_up(const uint16_t *xg, const uint16_t *w1, const float *b1g, const float *b1u,
                           const DispatchBuffers &d, uint16_t *act, int H, int IM, int E, float limit,
                           int mt_cap, hipStream_t s) {
-  return launch_gemm<CfgGateUp, true>(reinterpret_cast<const uint4 *>(xg),
-                                      reinterpret_cast<const uint4 *>(w1), b1g, b1u, d, act, H, IM,
-                                      E, limit, mt_cap, s);
+  return launch_gemm<CfgGemm, true>(reinterpret_cast<const uint4 *>(xg),
+                                    reinterpret_cast<const uint4 *>(w1), b1g, b1u, d, act, H, IM, E,
+                                    limit, mt_cap, s);
 }
 
 hipError_t launch_down(const uint16_t *act, const uint16_t *w2, const float *b2,
                        const DispatchBuffers &d, float *y, int H, int IM, int E, int mt_cap,
                        hipStream_t s) {
-  return launch_gemm<CfgDown, false>(reinterpret_cast<const uint4 *>(act),
+  return launch_gemm<CfgGemm, false>(reinterpret_cast<const uint4 *>(act),
                                      reinterpret_cast<const uint4 *>(w2), b2, nullptr, d, y, IM, H, E,
                                      0.f, mt_cap, s);
 }

@@ -14,15 +14,15 @@ constexpr int kRowBlock = 32;   // rows of one MFMA fragment (v_mfma_f32_32x32x1
 constexpr int kFragK = 16;      // reduction depth of one fragment
 constexpr int kFragBytes = 1024;  // 64 lanes x 8 bf16
 constexpr int kTileRows = 256;  // tallest row tile of the grouped GEMMs
-constexpr int kTileGran = 64;   // row tiles are multiples of this (2 wave rows x 32)
+constexpr int kTileGran = 32;   // row tiles are multiples of one row block
 constexpr float kAlpha = 1.702f;  // run.cpp:709
 
 // Per-expert record written by the scan kernel and read by the GEMMs.
 struct ExpertInfo {
-  int row0;       // first padded row of the expert's segment (multiple of 64)
+  int row0;       // first padded row of the expert's segment (multiple of 32)
   int rows;       // valid rows (assignments) of the expert
   int n_mt;       // number of row tiles
-  int rb;         // fragments per wave row in every tile of this expert (1..4)
+  int rb;         // row blocks in every tile of this expert (1..8)
   int tile_base;  // number of row tiles of all lower experts
   int pad_[3];
 };
