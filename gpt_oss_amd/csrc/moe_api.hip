@@ -199,7 +199,7 @@ int moe_create(const moe_config *cfg, moe_handle **out) {
     moe_destroy(h);
     return rc;
   }
-  h->layer_bytes = (size_t)h->E_pad * H * 8 + (size_t)h->E_pad * 4 +
+  h->layer_bytes = (size_t)h->E_pad * H * 2 + (size_t)h->E_pad * 4 +
                    (size_t)E * 2 * IM * H * 2 + (size_t)E * 2 * IM * 4 +
                    (size_t)E * H * IM * 2 + (size_t)E * H * 4;
   *out = h;

@@ -28,7 +28,7 @@ struct ExpertInfo {
 };
 
 struct LayerWeights {
-  double *wr = nullptr;    // router weight, f64 MFMA fragments
+  uint16_t *wr = nullptr;  // router weight, bf16 in the operand order of the f64 MFMA
   float *br = nullptr;     // router bias, padded experts = -inf
   uint16_t *w1 = nullptr;  // gate_up weight, bf16 MFMA fragments, gate/up blocks paired
   float *b1g = nullptr;    // gate bias [E, IM]
@@ -40,14 +40,14 @@ struct LayerWeights {
 
 // ---- kernel launchers (defined in the .hip files) ----
 
-hipError_t launch_pack_router(const float *w_src, const float *b_src, double *wr, float *br,
+hipError_t launch_pack_router(const float *w_src, const float *b_src, uint16_t *wr, float *br,
                               int E, int E_pad, int H, hipStream_t s);
 hipError_t launch_pack_weight(const float *src, uint16_t *dst, int rows, int cols, bool gate_up,
                               hipStream_t s);
 hipError_t launch_pack_bias(const float *src, float *dst_a, float *dst_b, int n, bool deinterleave,
                             hipStream_t s);
 
-hipError_t launch_router(const uint16_t *x, const int *pos, const double *wr, const float *br,
+hipError_t launch_router(const uint16_t *x, const int *pos, const uint16_t *wr, const float *br,
                          int T, int H, int E, int E_pad, float *score, int *topk_i, float *topk_v,
                          hipStream_t s);
 

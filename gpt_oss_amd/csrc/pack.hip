@@ -52,14 +52,16 @@ __global__ void pack_weight_kernel(const float *__restrict__ src, uint4 *__restr
   }
 }
 
-// Router weight as f64 fragments of v_mfma_f64_16x16x4_f64.  Order
-// [expert block of 16][k chunk of 32][lane][s], s = 0..7: lane l holds expert
-// 16*nb + (l % 16) and k = 32*kc + 8*(l / 16) + s.  The s-th MFMA of a chunk
-// multiplies these with the s-th of 8 consecutive activations a lane loaded.
+// Router weight in the operand order of v_mfma_f64_16x16x4_f64, kept as bf16
+// (the kernel widens to f64 on the fly: a quarter of the bytes of an f64 copy,
+// and the router is otherwise bound by streaming this matrix through every CU).
+// Order [expert block of 16][k chunk of 32][lane][s], s = 0..7: lane l holds
+// expert 16*nb + (l % 16) and k = 32*kc + 8*(l / 16) + s.  The s-th MFMA of a
+// chunk multiplies these with the s-th of 8 consecutive activations a lane loaded.
 // Experts beyond E are zero weight with bias -inf, so they are never selected.
 __global__ void pack_router_kernel(const float *__restrict__ w, const float *__restrict__ b,
-                                   double *__restrict__ wr, float *__restrict__ br, int E, int E_pad,
-                                   int H) {
+                                   uint16_t *__restrict__ wr, float *__restrict__ br, int E,
+                                   int E_pad, int H) {
   const int kc_total = H / 32;
   const size_t n = (size_t)(E_pad / 16) * kc_total * 64 * 8;
   for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n;
@@ -71,7 +73,7 @@ __global__ void pack_router_kernel(const float *__restrict__ w, const float *__r
     const int nb = (int)(f / kc_total);
     const int e = nb * 16 + (lane & 15);
     const int k = kc * 32 + 8 * (lane >> 4) + s;
-    wr[i] = e < E ? (double)bf16_round(w[(size_t)e * H + k]) : 0.0;
+    wr[i] = e < E ? f32_to_bf16_rne(w[(size_t)e * H + k]) : (uint16_t)0;
   }
   const int t = blockIdx.x * blockDim.x + threadIdx.x;
   if (t < E_pad) br[t] = t < E ? bf16_round(b[t]) : -INFINITY;
@@ -91,7 +93,7 @@ __global__ void pack_bias_kernel(const float *__restrict__ src, float *__restric
   }
 }
 
-hipError_t launch_pack_router(const float *w_src, const float *b_src, double *wr, float *br, int E,
+hipError_t launch_pack_router(const float *w_src, const float *b_src, uint16_t *wr, float *br, int E,
                               int E_pad, int H, hipStream_t s) {
   pack_router_kernel<<<512, 256, 0, s>>>(w_src, b_src, wr, br, E, E_pad, H);
   return hipGetLastError();

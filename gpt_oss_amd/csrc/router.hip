@@ -16,13 +16,25 @@ namespace moe {
 
 typedef double f64x4 __attribute__((ext_vector_type(4)));
 
+// 8 bf16 -> 8 doubles (exact).
+__device__ __forceinline__ void widen8(const uint4 v, double (&d)[8]) {
+  d[0] = (double)__uint_as_float(v.x << 16);
+  d[1] = (double)__uint_as_float(v.x & 0xffff0000u);
+  d[2] = (double)__uint_as_float(v.y << 16);
+  d[3] = (double)__uint_as_float(v.y & 0xffff0000u);
+  d[4] = (double)__uint_as_float(v.z << 16);
+  d[5] = (double)__uint_as_float(v.z & 0xffff0000u);
+  d[6] = (double)__uint_as_float(v.w << 16);
+  d[7] = (double)__uint_as_float(v.w & 0xffff0000u);
+}
+
 // One workgroup = 16 tokens x all experts.  Its WPC waves split the reduction
 // dimension in chunks of 32 (wave w takes chunks w, w+WPC, ...), each wave
 // keeps NT 16x16 accumulators, and the partial sums are added in wave order
 // through LDS.  NT = E_pad / 16.
 template <int NT, int WPC>
 __global__ __launch_bounds__(WPC * 64) void router_kernel(
-    const uint16_t *__restrict__ x, const int *__restrict__ pos, const double *__restrict__ wr,
+    const uint16_t *__restrict__ x, const int *__restrict__ pos, const uint16_t *__restrict__ wr,
     const float *__restrict__ br, int T, int H, int E, float *__restrict__ score,
     int *__restrict__ topk_i, float *__restrict__ topk_v) {
   constexpr int E_pad = NT * 16;
@@ -42,34 +54,43 @@ __global__ __launch_bounds__(WPC * 64) void router_kernel(
 #pragma unroll
   for (int n = 0; n < NT; n++) acc[n] = f64x4{0.0, 0.0, 0.0, 0.0};
 
+  // The loads of chunk c + WPC are issued before the MFMAs of chunk c: with few
+  // waves per SIMD nothing else would cover their latency.
   const uint16_t *xrow = x + (size_t)t_ld * H + g * 8;
-  for (int c = w; c < kc_total; c += WPC) {
-    const uint4 xv = *reinterpret_cast<const uint4 *>(xrow + c * 32);
-    double xd[8];
-    xd[0] = (double)__uint_as_float(xv.x << 16);
-    xd[1] = (double)__uint_as_float(xv.x & 0xffff0000u);
-    xd[2] = (double)__uint_as_float(xv.y << 16);
-    xd[3] = (double)__uint_as_float(xv.y & 0xffff0000u);
-    xd[4] = (double)__uint_as_float(xv.z << 16);
-    xd[5] = (double)__uint_as_float(xv.z & 0xffff0000u);
-    xd[6] = (double)__uint_as_float(xv.w << 16);
-    xd[7] = (double)__uint_as_float(xv.w & 0xffff0000u);
+  const uint16_t *wlane = wr + (size_t)lane * 8;
+  uint4 xv = make_uint4(0, 0, 0, 0), wv[NT];
+  if (w < kc_total) {
+    xv = *reinterpret_cast<const uint4 *>(xrow + w * 32);
 #pragma unroll
-    for (int n = 0; n < NT; n++) {
-      const double *wp = wr + (((size_t)n * kc_total + c) * 64 + lane) * 8;
-      const double2 w01 = *reinterpret_cast<const double2 *>(wp);
-      const double2 w23 = *reinterpret_cast<const double2 *>(wp + 2);
-      const double2 w45 = *reinterpret_cast<const double2 *>(wp + 4);
-      const double2 w67 = *reinterpret_cast<const double2 *>(wp + 6);
-      acc[n] = __builtin_amdgcn_mfma_f64_16x16x4f64(xd[0], w01.x, acc[n], 0, 0, 0);
-      acc[n] = __builtin_amdgcn_mfma_f64_16x16x4f64(xd[1], w01.y, acc[n], 0, 0, 0);
-      acc[n] = __builtin_amdgcn_mfma_f64_16x16x4f64(xd[2], w23.x, acc[n], 0, 0, 0);
-      acc[n] = __builtin_amdgcn_mfma_f64_16x16x4f64(xd[3], w23.y, acc[n], 0, 0, 0);
-      acc[n] = __builtin_amdgcn_mfma_f64_16x16x4f64(xd[4], w45.x, acc[n], 0, 0, 0);
-      acc[n] = __builtin_amdgcn_mfma_f64_16x16x4f64(xd[5], w45.y, acc[n], 0, 0, 0);
-      acc[n] = __builtin_amdgcn_mfma_f64_16x16x4f64(xd[6], w67.x, acc[n], 0, 0, 0);
-      acc[n] = __builtin_amdgcn_mfma_f64_16x16x4f64(xd[7], w67.y, acc[n], 0, 0, 0);
+    for (int n = 0; n < NT; n++)
+      wv[n] = *reinterpret_cast<const uint4 *>(wlane + ((size_t)n * kc_total + w) * 512);
+  }
+  for (int c = w; c < kc_total; c += WPC) {
+    const int cn = min(c + WPC, kc_total - 1);  // the last prefetch repeats a chunk and is dropped
+    const uint4 xn = *reinterpret_cast<const uint4 *>(xrow + cn * 32);
+    uint4 wn[NT];
+#pragma unroll
+    for (int n = 0; n < NT; n++)
+      wn[n] = *reinterpret_cast<const uint4 *>(wlane + ((size_t)n * kc_total + cn) * 512);
+    double xd[8];
+    widen8(xv, xd);
+    // Two accumulators are advanced alternately so that back-to-back MFMAs do
+    // not depend on each other.
+    constexpr int NP = NT > 1 ? 2 : 1;
+#pragma unroll
+    for (int n = 0; n < NT; n += NP) {
+      double wd[NP][8];
+#pragma unroll
+      for (int p = 0; p < NP; p++) widen8(wv[n + p], wd[p]);
+#pragma unroll
+      for (int s = 0; s < 8; s++)
+#pragma unroll
+        for (int p = 0; p < NP; p++)
+          acc[n + p] = __builtin_amdgcn_mfma_f64_16x16x4f64(xd[s], wd[p][s], acc[n + p], 0, 0, 0);
     }
+    xv = xn;
+#pragma unroll
+    for (int n = 0; n < NT; n++) wv[n] = wn[n];
   }
 
 #pragma unroll
@@ -156,30 +177,19 @@ __global__ __launch_bounds__(WPC * 64) void router_kernel(
 }
 
 template <int NT>
-static hipError_t launch_router_nt(const uint16_t *x, const int *pos, const double *wr,
+static hipError_t launch_router_nt(const uint16_t *x, const int *pos, const uint16_t *wr,
                                    const float *br, int T, int H, int E, float *score, int *topk_i,
                                    float *topk_v, hipStream_t s) {
   const int grid = (T + 15) / 16;
-  // More waves per workgroup (a finer split of the reduction) when there are
-  // too few token tiles to occupy the 1024 SIMDs; bounded by the LDS the
-  // partial sums need (WPC * NT * 2 KB).
-  if constexpr (NT <= 2) {
-    if (grid < 128) {
-      router_kernel<NT, 16><<<grid, 16 * 64, 0, s>>>(x, pos, wr, br, T, H, E, score, topk_i, topk_v);
-      return hipGetLastError();
-    }
-  }
-  if constexpr (NT <= 4) {
-    if (grid < 256) {
-      router_kernel<NT, 8><<<grid, 8 * 64, 0, s>>>(x, pos, wr, br, T, H, E, score, topk_i, topk_v);
-      return hipGetLastError();
-    }
-  }
-  router_kernel<NT, 4><<<grid, 4 * 64, 0, s>>>(x, pos, wr, br, T, H, E, score, topk_i, topk_v);
+  // As many waves per workgroup (i.e. as fine a split of the reduction) as the
+  // LDS for the partial sums allows (WPC * NT * 2 KB <= 64 KB): more waves per
+  // SIMD hide the load latency, and small batches still occupy the SIMDs.
+  constexpr int WPC = NT <= 2 ? 16 : (NT <= 4 ? 8 : (NT <= 8 ? 4 : 2));
+  router_kernel<NT, WPC><<<grid, WPC * 64, 0, s>>>(x, pos, wr, br, T, H, E, score, topk_i, topk_v);
   return hipGetLastError();
 }
 
-hipError_t launch_router(const uint16_t *x, const int *pos, const double *wr, const float *br, int T,
+hipError_t launch_router(const uint16_t *x, const int *pos, const uint16_t *wr, const float *br, int T,
                          int H, int E, int E_pad, float *score, int *topk_i, float *topk_v,
                          hipStream_t s) {
   if (T <= 0) return hipSuccess;
