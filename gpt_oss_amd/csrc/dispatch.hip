@@ -56,9 +56,10 @@ __device__ __forceinline__ int block_exclusive_scan_256(int v, int *buf, int tid
 
 // Pass 2 (one workgroup): turns the per-workgroup counts into exclusive bases,
 // and builds per-expert offsets and the row-tile plan of the grouped GEMMs.
-// An expert with M rows gets n_mt = ceil(M / 256) tiles of equal height
-// 32 * rb, rb = ceil(M / (32 * n_mt)) in 1..8; its segment in the padded row
-// space is n_mt * 32 * rb rows long, so tiles never overlap the next expert.
+// An expert with M rows has ceil(M / 32) row blocks, cut into n_mt = ceil(row
+// blocks / 8) tiles as evenly as they go: the first `extra` tiles are rb + 1
+// row blocks high, the others rb.  Its segment in the padded row space is its
+// row blocks and no more, so an expert pads to at most 31 rows.
 __global__ __launch_bounds__(256) void dispatch_scan_kernel(int *__restrict__ blk_counts, int n_blk,
                                                            int E, int *__restrict__ offsets,
                                                            ExpertInfo *__restrict__ info,
@@ -73,9 +74,12 @@ __global__ __launch_bounds__(256) void dispatch_scan_kernel(int *__restrict__ bl
       count += c;
     }
   }
-  const int n_mt = (count + kTileRows - 1) / kTileRows;
-  const int rb = n_mt ? (count + kTileGran * n_mt - 1) / (kTileGran * n_mt) : 0;
-  const int padded = n_mt * rb * kTileGran;
+  const int n_rb = (count + kRowBlock - 1) / kRowBlock;
+  constexpr int kTileRb = kTileRows / kRowBlock;
+  const int n_mt = (n_rb + kTileRb - 1) / kTileRb;
+  const int rb = n_mt ? n_rb / n_mt : 0;
+  const int extra = n_mt ? n_rb - rb * n_mt : 0;
+  const int padded = n_rb * kRowBlock;
   int tot_count, tot_pad, tot_mt;
   const int ex_count = block_exclusive_scan_256(count, buf, e, &tot_count);
   const int ex_pad = block_exclusive_scan_256(padded, buf, e, &tot_pad);
@@ -88,7 +92,8 @@ __global__ __launch_bounds__(256) void dispatch_scan_kernel(int *__restrict__ bl
     inf.n_mt = n_mt;
     inf.rb = rb;
     inf.tile_base = ex_mt;
-    inf.pad_[0] = inf.pad_[1] = inf.pad_[2] = 0;
+    inf.extra = extra;
+    inf.pad_[0] = inf.pad_[1] = 0;
     info[e] = inf;
   }
   if (e == 0) {
@@ -223,10 +228,10 @@ __global__ __launch_bounds__(256) void combine_kernel(const float *__restrict__ 
 hipError_t launch_dispatch(const int *topk_i, const int *pos, int T, int E, const DispatchBuffers &d,
                            hipStream_t s) {
   const int n_blk = (T + kDispThreads - 1) / kDispThreads;
-  // Rows of the padded space this batch can reach: sum over experts of
-  // n_mt * 64 * rb < 1.25 * A + 64 * E.
+  // Rows of the padded space this batch can reach: every expert rounds its
+  // rows up to a multiple of 32.
   const long long A = (long long)T * kTopK;
-  const long long reach = A + A / 4 + (long long)kTileGran * E;
+  const long long reach = A + (long long)kTileGran * E;
   const int fill_rows = (int)(reach < d.a_pad_cap ? reach : d.a_pad_cap);
   dispatch_count_kernel<<<n_blk, kDispThreads, 0, s>>>(topk_i, pos, T, E, d.blk_counts, d.rowmap,
                                                        fill_rows, d.perm);

@@ -12,8 +12,8 @@
 // Tiling.  A workgroup of NW waves owns a tile of (RBT*32) rows x
 // (NW*NBW*32) columns of one expert.  The waves split the columns only: each
 // wave keeps RBT x NBW accumulators of 32x32 over all rows of the tile, RBT =
-// 1..8 following the expert's row count (ExpertInfo::rb), so ragged segments
-// pad to at most 31 rows per tile and MFMA work follows the real rows.
+// 1..8 following the expert's row count (see dispatch_scan_kernel), so a ragged
+// segment pads to at most 31 rows and MFMA work follows the real rows.
 //
 // Feeding the matrix cores.  What bounds this kernel is how fast one CU can
 // take data in from L2 (about 45 GB/s with 100 KB in flight, 55-60 GB/s with
@@ -93,8 +93,8 @@ __device__ __forceinline__ bool locate_tile(const ExpertInfo *__restrict__ info,
   const int mt = rem % inf.n_mt;
   tc.e = e;
   tc.nt = rem / inf.n_mt;
-  rb = inf.rb;
-  tc.rows0 = mt * rb * kRowBlock;
+  rb = inf.rb + (mt < inf.extra ? 1 : 0);
+  tc.rows0 = (mt * inf.rb + min(mt, inf.extra)) * kRowBlock;
   tc.rb0 = (inf.row0 + tc.rows0) / kRowBlock;
   return true;
 }
@@ -137,6 +137,8 @@ struct GemmCfg {
   static constexpr int TILE_NB = NW * NBW;              // column blocks per tile
   static constexpr int RBT_MAX = kTileRows / kRowBlock;  // row blocks per tile, at most
   static constexpr int STAGE = RBT_MAX * KPS * 64;       // uint4 per LDS stage (16 KB)
+  static constexpr int EPI_LD = NBW * 32 + 8;            // floats per buffered output row
+  static constexpr int EPI_WAVE = 32 * EPI_LD / 4;       // uint4 per wave of epilogue buffer
 };
 
 template <int RBT, typename C, bool GATE_UP>
@@ -153,7 +155,12 @@ __device__ __forceinline__ void gemm_tile(const uint4 *__restrict__ a_frag,  // 
                                           uint4 *__restrict__ s0, uint4 *__restrict__ s1,
                                           uint4 *__restrict__ s2, uint4 *__restrict__ s3,
                                           uint4 *__restrict__ s4, uint4 *__restrict__ s5,
-                                          uint4 *__restrict__ s6) {
+                                          uint4 *__restrict__ s6,
+                                          // The epilogue buffers are not carved out of the
+                                          // ring: the compiler would make every read of them
+                                          // wait for all outstanding vector memory operations,
+                                          // the epilogue's own stores included.
+                                          uint4 *__restrict__ epi) {
   StageRing<C::R> ring;
   ring.p[0] = s0; ring.p[1] = s1; ring.p[2] = s2; ring.p[3] = s3;
   ring.p[4] = s4; ring.p[5] = s5; ring.p[6] = s6;
@@ -315,12 +322,10 @@ __device__ __forceinline__ void gemm_tile(const uint4 *__restrict__ a_frag,  // 
 #undef MOE_WAIT_STEPS
 
   // Epilogue.  Accumulator register q of lane l is row 8*(q/4) + 4*(l/32) + q%4,
-  // column l % 32 of its 32x32 block.  Results are re-ordered through LDS (the
-  // ring is idle now; each wave takes a stage of its own) so that they leave as
-  // 16 bytes per lane, 1 KB contiguous per wave store.
-  lds_barrier();  // every wave has finished reading the stages
-  static_assert(NW <= R, "one stage per wave serves as its epilogue buffer");
-  uint4 *ebuf = ring.p[w];
+  // column l % 32 of its 32x32 block.  Results are re-ordered through this
+  // wave's piece of LDS so that they leave as 16 bytes per lane, 1 KB contiguous
+  // per wave store.
+  uint4 *ebuf = epi + w * C::EPI_WAVE;
   const int n = lane & 31;
   const int rsub = 4 * (lane >> 5);
   if (w * NBW >= nb_valid) return;  // a wave without columns (last column tile only)
@@ -331,7 +336,7 @@ __device__ __forceinline__ void gemm_tile(const uint4 *__restrict__ a_frag,  // 
     // order the down GEMM reads as its row operand: column j is k block j/16,
     // lane ((j%16)/8)*32 + row, element j % 8.
     static_assert(NBW % 2 == 0, "gate and up blocks of a pair must sit in one wave");
-    static_assert(NBW * 64 <= C::STAGE, "epilogue buffer");
+    static_assert(NBW * 64 <= C::EPI_WAVE, "epilogue buffer");
     uint4 *act = reinterpret_cast<uint4 *>(outp);
     uint16_t *e16 = reinterpret_cast<uint16_t *>(ebuf);
     const int kb2_total = out_ld / kFragK;
@@ -366,8 +371,7 @@ __device__ __forceinline__ void gemm_tile(const uint4 *__restrict__ a_frag,  // 
       }
     }
   } else {
-    constexpr int LD = NBW * 32 + 8;  // floats per buffered row; +8 keeps the two lane halves on different banks
-    static_assert(32 * LD * 4 <= C::STAGE * 16, "epilogue buffer");
+    constexpr int LD = C::EPI_LD;  // +8 floats keep the two lane halves on different banks
     float *y = reinterpret_cast<float *>(outp);
     float *ef = reinterpret_cast<float *>(ebuf);
     float bb[NBW];
@@ -408,6 +412,7 @@ __global__ __launch_bounds__(C::THREADS) void grouped_gemm_kernel(
   static_assert(R == 7, "seven stage arrays are declared below");
   __shared__ uint4 st0[C::STAGE], st1[C::STAGE], st2[C::STAGE], st3[C::STAGE], st4[C::STAGE],
       st5[C::STAGE], st6[C::STAGE];
+  __shared__ uint4 epi[C::NW * C::EPI_WAVE];
   const int KB = K / kFragK;
   const int nb_total = (GATE_UP ? 2 * N : N) / kRowBlock;  // weight row blocks per expert
   const int n_ct = (nb_total + C::TILE_NB - 1) / C::TILE_NB;
@@ -420,11 +425,11 @@ __global__ __launch_bounds__(C::THREADS) void grouped_gemm_kernel(
   const float *ba = bias_a + (size_t)tc.e * N;
   const float *bb = GATE_UP ? bias_b + (size_t)tc.e * N : nullptr;
 #define MOE_TILE_CASE(n) \
-  case n: gemm_tile<n, C, GATE_UP>(a_frag, b_frag, KB, tc.rb0, nb0, nb_valid, ba, bb, outp, N, limit, st0, st1, st2, st3, st4, st5, st6); break;
+  case n: gemm_tile<n, C, GATE_UP>(a_frag, b_frag, KB, tc.rb0, nb0, nb_valid, ba, bb, outp, N, limit, st0, st1, st2, st3, st4, st5, st6, epi); break;
   switch (rb) {
     MOE_TILE_CASE(1) MOE_TILE_CASE(2) MOE_TILE_CASE(3) MOE_TILE_CASE(4)
     MOE_TILE_CASE(5) MOE_TILE_CASE(6) MOE_TILE_CASE(7)
-    default: gemm_tile<8, C, GATE_UP>(a_frag, b_frag, KB, tc.rb0, nb0, nb_valid, ba, bb, outp, N, limit, st0, st1, st2, st3, st4, st5, st6); break;
+    default: gemm_tile<8, C, GATE_UP>(a_frag, b_frag, KB, tc.rb0, nb0, nb_valid, ba, bb, outp, N, limit, st0, st1, st2, st3, st4, st5, st6, epi); break;
   }
 #undef MOE_TILE_CASE
 }

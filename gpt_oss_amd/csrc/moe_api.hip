@@ -123,7 +123,7 @@ int run_experts(moe_handle *h, int layer, const uint16_t *x, const int *pos, con
   const LayerWeights &lw = h->layers[layer];
   const int A = T * kTopK;
   const int mt_cap = A / kTileRows + c.experts;
-  const int rb_cap = (A + A / 4 + kTileGran * c.experts + kRowBlock - 1) / kRowBlock;
+  const int rb_cap = (A + kTileGran * c.experts + kRowBlock - 1) / kRowBlock;
   HIP_TRY(tm.mark(MOE_STAGE_DISPATCH));
   HIP_TRY(launch_dispatch(topk_i, pos, T, c.experts, h->disp, s));
   HIP_TRY(tm.mark(MOE_STAGE_GATHER));
@@ -176,7 +176,7 @@ int moe_create(const moe_config *cfg, moe_handle **out) {
 
   const int E = cfg->experts, H = cfg->hidden, IM = cfg->inter, T = cfg->max_tokens;
   h->a_cap = T * kTopK;
-  h->a_pad_cap = ((h->a_cap + h->a_cap / 4 + kTileGran * E + kTileGran - 1) / kTileGran) * kTileGran;
+  h->a_pad_cap = ((h->a_cap + kTileGran * E + kTileGran - 1) / kTileGran) * kTileGran;
   h->n_blk_cap = (T + 255) / 256;
   int rc = MOE_OK;
 #define ALLOC(ptr, count)                                   \

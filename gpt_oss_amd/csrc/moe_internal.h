@@ -14,7 +14,7 @@ constexpr int kRowBlock = 32;   // rows of one MFMA fragment (v_mfma_f32_32x32x1
 constexpr int kFragK = 16;      // reduction depth of one fragment
 constexpr int kFragBytes = 1024;  // 64 lanes x 8 bf16
 constexpr int kTileRows = 256;  // tallest row tile of the grouped GEMMs
-constexpr int kTileGran = 32;   // row tiles are multiples of one row block
+constexpr int kTileGran = 32;   // an expert's segment of padded rows is a multiple of one row block
 constexpr float kAlpha = 1.702f;  // run.cpp:709
 
 // Per-expert record written by the scan kernel and read by the GEMMs.
@@ -22,9 +22,10 @@ struct ExpertInfo {
   int row0;       // first padded row of the expert's segment (multiple of 32)
   int rows;       // valid rows (assignments) of the expert
   int n_mt;       // number of row tiles
-  int rb;         // row blocks in every tile of this expert (1..8)
+  int rb;         // row blocks of the expert's shorter tiles (0..8)
   int tile_base;  // number of row tiles of all lower experts
-  int pad_[3];
+  int extra;      // its first `extra` tiles have rb + 1 row blocks
+  int pad_[2];
 };
 
 struct LayerWeights {
