@@ -49,12 +49,25 @@ __device__ __forceinline__ uint16_t f32_to_bf16_rne_dev(float f) {
   return (uint16_t)(u >> 16);
 }
 
-// run.cpp:709-726: gate clamped from above, up clamped on both sides.
-__device__ __forceinline__ float swiglu(float g, float u, float limit) {
+// run.cpp:709-726: gate clamped from above, up clamped on both sides, then
+// gate * sigmoid(alpha * gate) * (up + 1).  u1 is up + 1 already (the 1 rides
+// in the accumulator's start value together with the bias).
+__device__ __forceinline__ float swiglu_shifted(float g, float u1, float limit) {
+  constexpr float kNegAlphaLog2e = -kAlpha * 1.4426950408889634f;
   g = fminf(g, limit);
-  u = fminf(fmaxf(u, -limit), limit);
-  const float s = __builtin_amdgcn_rcpf(1.0f + __expf(-kAlpha * g));
-  return g * s * (u + 1.0f);
+  u1 = __builtin_amdgcn_fmed3f(u1, 1.0f - limit, 1.0f + limit);
+  const float s = __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(kNegAlphaLog2e * g));
+  return g * s * u1;
+}
+
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+// two floats -> packed bf16, round to nearest even (v_cvt_pk_bf16_f32); a in the low half
+__device__ __forceinline__ uint32_t pack_bf16(float a, float b) {
+  f32x2 v = {a, b};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));
 }
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
@@ -177,13 +190,35 @@ __device__ __forceinline__ void gemm_tile(const uint4 *__restrict__ a_frag,  // 
   const int lane = tid & 63;
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
 
-  f32x16 acc[RBT][NBW];
+  // The accumulators start from the bias (the up half of gate_up from bias + 1,
+  // see swiglu_shifted).  gate_up computes the transposed product (weights as
+  // the MFMA's first operand): register q of lane l is then weight row
+  // 8*(q/4) + 4*(l/32) + q%4 of its block and token l % 32.  down computes the
+  // product as it is: register q is token 8*(q/4) + 4*(l/32) + q%4, lane l
+  // column l % 32.  The bias loads go out first and are consumed after the
+  // pipeline's loads have been issued.
+  static_assert(!GATE_UP || NBW % 2 == 0, "gate and up blocks of a pair must sit in one wave");
+  float4 bias_g[NBW / 2 + 1][4], bias_u[NBW / 2 + 1][4];
+  float bias_d[NBW];
+  if (GATE_UP) {
+    const int pairs_valid = max(1, (nb_valid - w * NBW) >> 1);
+    const int P0 = (nb0 + w * NBW) >> 1;
 #pragma unroll
-  for (int i = 0; i < RBT; i++)
+    for (int p = 0; p < NBW / 2; p++) {
+      const int P = P0 + min(p, pairs_valid - 1);
+#pragma unroll
+      for (int g = 0; g < 4; g++) {
+        const int j = kRowBlock * P + 8 * g + 4 * (lane >> 5);
+        bias_g[p][g] = *reinterpret_cast<const float4 *>(bias_a + j);
+        bias_u[p][g] = *reinterpret_cast<const float4 *>(bias_b + j);
+      }
+    }
+  } else {
 #pragma unroll
     for (int j = 0; j < NBW; j++)
-#pragma unroll
-      for (int q = 0; q < 16; q++) acc[i][j][q] = 0.f;
+      bias_d[j] = bias_a[kRowBlock * (nb0 + min(w * NBW + j, nb_valid - 1)) + (lane & 31)];
+  }
+  f32x16 acc[RBT][NBW];
 
   const uint4 *a_src = a_frag + (size_t)rb0 * KB * 64 + lane;
   // Column blocks past the end of the matrix (last column tile only) re-load
@@ -209,6 +244,11 @@ __device__ __forceinline__ void gemm_tile(const uint4 *__restrict__ a_frag,  // 
   auto read_a = [&](const uint4 *st, int kk, int buf, int i) {
     fa[buf][i] = __builtin_bit_cast(bf16x8, st[(i * KPS + kk) * 64 + lane]);
   };
+  auto mma = [](bf16x8 rows, u32x4 cols, f32x16 c) {
+    const bf16x8 colv = __builtin_bit_cast(bf16x8, cols);
+    return GATE_UP ? __builtin_amdgcn_mfma_f32_32x32x16_bf16(colv, rows, c, 0, 0, 0)
+                   : __builtin_amdgcn_mfma_f32_32x32x16_bf16(rows, colv, c, 0, 0, 0);
+  };
   // "all but the newest k steps have landed", k = 0 .. R-2
 #define MOE_WAIT_STEPS(k)                            \
   switch (k) {                                       \
@@ -232,6 +272,27 @@ __device__ __forceinline__ void gemm_tile(const uint4 *__restrict__ a_frag,  // 
 #pragma unroll
       for (int m = 0; m < LB; m++) issue_b(s, s, m);
     }
+  }
+  if (GATE_UP) {
+#pragma unroll
+    for (int p = 0; p < NBW / 2; p++)
+#pragma unroll
+      for (int g = 0; g < 4; g++)
+#pragma unroll
+        for (int i = 0; i < RBT; i++) {
+          const float4 bg = bias_g[p][g], bu = bias_u[p][g];
+          acc[i][2 * p][4 * g + 0] = bg.x; acc[i][2 * p][4 * g + 1] = bg.y;
+          acc[i][2 * p][4 * g + 2] = bg.z; acc[i][2 * p][4 * g + 3] = bg.w;
+          acc[i][2 * p + 1][4 * g + 0] = bu.x + 1.0f; acc[i][2 * p + 1][4 * g + 1] = bu.y + 1.0f;
+          acc[i][2 * p + 1][4 * g + 2] = bu.z + 1.0f; acc[i][2 * p + 1][4 * g + 3] = bu.w + 1.0f;
+        }
+  } else {
+#pragma unroll
+    for (int j = 0; j < NBW; j++)
+#pragma unroll
+      for (int i = 0; i < RBT; i++)
+#pragma unroll
+        for (int q = 0; q < 16; q++) acc[i][j][q] = bias_d[j];
   }
   if (R - 1 < n_steps) {
 #pragma unroll
@@ -267,9 +328,7 @@ __device__ __forceinline__ void gemm_tile(const uint4 *__restrict__ a_frag,  // 
           if (refill_b) issue_b((u + R - 1) % R, ks + R - 1, t - RBT);
         }
       }
-      acc[m / NBW][m % NBW] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-          fa[0][m / NBW], __builtin_bit_cast(bf16x8, bq[u][(m % NBW) * KPS + 0]),
-          acc[m / NBW][m % NBW], 0, 0, 0);
+      acc[m / NBW][m % NBW] = mma(fa[0][m / NBW], bq[u][(m % NBW) * KPS + 0], acc[m / NBW][m % NBW]);
       __builtin_amdgcn_sched_barrier(0);
     }
     const bool more = STEADY || ks + 1 < n_steps;
@@ -294,9 +353,7 @@ __device__ __forceinline__ void gemm_tile(const uint4 *__restrict__ a_frag,  // 
           if (more) read_a(nxt, 0, 0, t - LA);
         }
       }
-      acc[m / NBW][m % NBW] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-          fa[1][m / NBW], __builtin_bit_cast(bf16x8, bq[u][(m % NBW) * KPS + 1]),
-          acc[m / NBW][m % NBW], 0, 0, 0);
+      acc[m / NBW][m % NBW] = mma(fa[1][m / NBW], bq[u][(m % NBW) * KPS + 1], acc[m / NBW][m % NBW]);
       __builtin_amdgcn_sched_barrier(0);
     }
   };
@@ -321,63 +378,51 @@ __device__ __forceinline__ void gemm_tile(const uint4 *__restrict__ a_frag,  // 
   }
 #undef MOE_WAIT_STEPS
 
-  // Epilogue.  Accumulator register q of lane l is row 8*(q/4) + 4*(l/32) + q%4,
-  // column l % 32 of its 32x32 block.  Results are re-ordered through this
-  // wave's piece of LDS so that they leave as 16 bytes per lane, 1 KB contiguous
-  // per wave store.
-  uint4 *ebuf = epi + w * C::EPI_WAVE;
-  const int n = lane & 31;
-  const int rsub = 4 * (lane >> 5);
+  // Epilogue.
   if (w * NBW >= nb_valid) return;  // a wave without columns (last column tile only)
   if (GATE_UP) {
     // Column blocks come in (gate, up) pairs (see pack_weight_kernel): blocks 2P
     // and 2P+1 of the product hold gate_j and up_j of j = 32P .. 32P+31 in the
     // same lane and register.  The activation goes out as bf16 in the fragment
     // order the down GEMM reads as its row operand: column j is k block j/16,
-    // lane ((j%16)/8)*32 + row, element j % 8.
-    static_assert(NBW % 2 == 0, "gate and up blocks of a pair must sit in one wave");
-    static_assert(NBW * 64 <= C::EPI_WAVE, "epilogue buffer");
+    // lane ((j%16)/8)*32 + token, element j % 8.  Registers 4g .. 4g+3 of lane
+    // (token t, half h) are j = 8g + 4h .. +3: elements 4h .. 4h+3 of the
+    // fragment lane (g % 2)*32 + t of k block g / 2.  One exchange between the
+    // lane halves (v_permlane32_swap) per dword completes the 16 bytes of every
+    // fragment lane; nothing goes through LDS.
     uint4 *act = reinterpret_cast<uint4 *>(outp);
-    uint16_t *e16 = reinterpret_cast<uint16_t *>(ebuf);
     const int kb2_total = out_ld / kFragK;
-    const int P0 = (nb0 + w * NBW) >> 1;              // first pair of this wave
+    const int P0 = (nb0 + w * NBW) >> 1;                // first pair of this wave
     const int pairs_valid = (nb_valid - w * NBW) >> 1;  // >= 1 here
-    float bg[NBW / 2], bu[NBW / 2];
-#pragma unroll
-    for (int p = 0; p < NBW / 2; p++) {
-      const int P = P0 + min(p, pairs_valid - 1);
-      bg[p] = bias_a[kRowBlock * P + n];
-      bu[p] = bias_b[kRowBlock * P + n];
-    }
-    // element offset of (row 0, column n of pair p) inside the wave's buffer of NBW fragments
-    const int e_off = ((n >> 4) * 64 + ((n & 15) >> 3) * 32) * 8 + (n & 7);
 #pragma unroll
     for (int i = 0; i < RBT; i++) {
 #pragma unroll
       for (int p = 0; p < NBW / 2; p++) {
-        uint16_t *dst = e16 + p * 2 * 64 * 8 + e_off;
+        uint32_t pk[4][2];
 #pragma unroll
-        for (int q = 0; q < 16; q++) {
-          const int r = 8 * (q >> 2) + rsub + (q & 3);
-          dst[r * 8] = f32_to_bf16_rne_dev(
-              swiglu(acc[i][2 * p][q] + bg[p], acc[i][2 * p + 1][q] + bu[p], limit));
+        for (int g = 0; g < 4; g++)
+#pragma unroll
+          for (int d = 0; d < 2; d++)
+            pk[g][d] = pack_bf16(
+                swiglu_shifted(acc[i][2 * p][4 * g + 2 * d], acc[i][2 * p + 1][4 * g + 2 * d], limit),
+                swiglu_shifted(acc[i][2 * p][4 * g + 2 * d + 1], acc[i][2 * p + 1][4 * g + 2 * d + 1],
+                               limit));
+        uint4 *dst = act + ((size_t)(rb0 + i) * kb2_total + 2 * (P0 + p)) * 64 + lane;
+#pragma unroll
+        for (int kb = 0; kb < 2; kb++) {
+          // upper lane half of registers 8kb .. 8kb+3 <-> lower lane half of 8kb+4 .. 8kb+7
+          const u32x2 s0 = __builtin_amdgcn_permlane32_swap(pk[2 * kb][0], pk[2 * kb + 1][0], false, false);
+          const u32x2 s1 = __builtin_amdgcn_permlane32_swap(pk[2 * kb][1], pk[2 * kb + 1][1], false, false);
+          if (p < pairs_valid) dst[kb * 64] = make_uint4(s0[0], s1[0], s0[1], s1[1]);
         }
-      }
-      uint4 *row_dst = act + ((size_t)(rb0 + i) * kb2_total + 2 * P0) * 64 + lane;
-#pragma unroll
-      for (int f = 0; f < NBW; f++) {
-        const uint4 v = ebuf[f * 64 + lane];
-        if ((f >> 1) < pairs_valid) row_dst[f * 64] = v;
       }
     }
   } else {
     constexpr int LD = C::EPI_LD;  // +8 floats keep the two lane halves on different banks
     float *y = reinterpret_cast<float *>(outp);
-    float *ef = reinterpret_cast<float *>(ebuf);
-    float bb[NBW];
-#pragma unroll
-    for (int j = 0; j < NBW; j++)
-      bb[j] = bias_a[kRowBlock * (nb0 + min(w * NBW + j, nb_valid - 1)) + n];
+    float *ef = reinterpret_cast<float *>(epi + w * C::EPI_WAVE);
+    const int n = lane & 31;
+    const int rsub = 4 * (lane >> 5);
     const int col0 = kRowBlock * (nb0 + w * NBW);
 #pragma unroll
     for (int i = 0; i < RBT; i++) {
@@ -386,7 +431,7 @@ __device__ __forceinline__ void gemm_tile(const uint4 *__restrict__ a_frag,  // 
 #pragma unroll
         for (int q = 0; q < 16; q++) {
           const int r = 8 * (q >> 2) + rsub + (q & 3);
-          ef[r * LD + 32 * j + n] = acc[i][j][q] + bb[j];
+          ef[r * LD + 32 * j + n] = acc[i][j][q];
         }
       const size_t row0 = (size_t)(rb0 + i) * kRowBlock;
 #pragma unroll
