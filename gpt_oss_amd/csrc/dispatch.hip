@@ -60,11 +60,19 @@ __device__ __forceinline__ int block_exclusive_scan_256(int v, int *buf, int tid
 // blocks / 8) tiles as evenly as they go: the first `extra` tiles are rb + 1
 // row blocks high, the others rb.  Its segment in the padded row space is its
 // row blocks and no more, so an expert pads to at most 31 rows.
+//
+// It also cuts the tile sequence of either GEMM (n_ct column tiles per row
+// tile) into the 8 ranges of the XCDs, by estimated cost: a tile of r row blocks
+// costs kCostPerTile + kCostPerRowBlock * r.
 __global__ __launch_bounds__(256) void dispatch_scan_kernel(int *__restrict__ blk_counts, int n_blk,
-                                                           int E, int *__restrict__ offsets,
+                                                           int E, int n_ct_gate_up, int n_ct_down,
+                                                           int *__restrict__ offsets,
                                                            ExpertInfo *__restrict__ info,
                                                            int *__restrict__ totals) {
   __shared__ int buf[256];
+  __shared__ int sh_cost[257];   // exclusive prefix of the experts' cost per column tile
+  __shared__ int sh_tiles[257];  // exclusive prefix of their row tiles
+  __shared__ int sh_bound[2][kXcds + 1];
   const int e = threadIdx.x;
   int count = 0;
   if (e < E) {
@@ -96,12 +104,70 @@ __global__ __launch_bounds__(256) void dispatch_scan_kernel(int *__restrict__ bl
     inf.pad_[0] = inf.pad_[1] = 0;
     info[e] = inf;
   }
+  // cost of one column tile's worth of the expert's row tiles
+  const int cost = n_mt * (kCostPerTile + kCostPerRowBlock * rb) + kCostPerRowBlock * extra;
+  int tot_cost;
+  const int ex_cost = block_exclusive_scan_256(cost, buf, e, &tot_cost);
+  sh_cost[e] = ex_cost;
+  sh_tiles[e] = ex_mt;
   if (e == 0) {
+    sh_cost[256] = tot_cost;
+    sh_tiles[256] = tot_mt;
     offsets[E] = tot_count;
-    totals[0] = tot_mt;
-    totals[1] = tot_pad;
-    totals[2] = tot_count;
+    totals[kTotTiles] = tot_mt;
+    totals[kTotRows] = tot_pad;
+    totals[kTotAssign] = tot_count;
     totals[3] = 0;
+  }
+  __syncthreads();
+  // Thread (g, x): boundary x of GEMM g = first tile at which the cost so far
+  // reaches x/8 of the total.  Tile L = (expert, column tile, row tile).
+  if (e < 2 * (kXcds + 1)) {
+    const int g = e / (kXcds + 1), x = e % (kXcds + 1);
+    const int n_ct = g ? n_ct_down : n_ct_gate_up;
+    const int total_tiles = tot_mt * n_ct;
+    int bound;
+    if (x == 0) {
+      bound = 0;
+    } else if (x == kXcds) {
+      bound = total_tiles;
+    } else {
+      const long long target = (long long)tot_cost * n_ct * x / kXcds;
+      // last expert whose first tile starts at or before the target
+      int lo = 0, hi = 255;
+      while (lo < hi) {
+        const int mid = (lo + hi + 1) >> 1;
+        if ((long long)sh_cost[mid] * n_ct <= target) lo = mid; else hi = mid - 1;
+      }
+      const int c_e = sh_cost[lo + 1] - sh_cost[lo];  // > 0: the search stops on an expert with tiles
+      const int m_e = sh_tiles[lo + 1] - sh_tiles[lo];
+      long long rest = target - (long long)sh_cost[lo] * n_ct;
+      const int ct = c_e ? (int)(rest / c_e) : 0;
+      rest -= (long long)ct * c_e;
+      // row tiles inside the column tile: average cost is close enough
+      const int mt = c_e ? (int)(rest * m_e / c_e) : 0;
+      bound = sh_tiles[lo] * n_ct + min(ct, n_ct) * m_e + min(mt, m_e);
+      bound = min(bound, total_tiles);
+    }
+    sh_bound[g][x] = bound;
+  }
+  __syncthreads();
+  // keep every range within what the launch grid provides for (xcd_tile_cap)
+  if (e < 2) {
+    const int n_ct = e ? n_ct_down : n_ct_gate_up;
+    const int total_tiles = tot_mt * n_ct;
+    const int cap = xcd_tile_cap(total_tiles);
+    int *out = totals + (e ? kTotBoundsDown : kTotBoundsGateUp);
+    int prev = 0;
+    out[0] = 0;
+    for (int x = 1; x < kXcds; x++) {
+      int bnd = sh_bound[e][x];
+      bnd = max(bnd, max(prev, total_tiles - (kXcds - x) * cap));
+      bnd = min(bnd, prev + cap);
+      out[x] = bnd;
+      prev = bnd;
+    }
+    out[kXcds] = total_tiles;
   }
 }
 
@@ -225,8 +291,8 @@ __global__ __launch_bounds__(256) void combine_kernel(const float *__restrict__ 
   }
 }
 
-hipError_t launch_dispatch(const int *topk_i, const int *pos, int T, int E, const DispatchBuffers &d,
-                           hipStream_t s) {
+hipError_t launch_dispatch(const int *topk_i, const int *pos, int T, int E, int n_ct_gate_up,
+                           int n_ct_down, const DispatchBuffers &d, hipStream_t s) {
   const int n_blk = (T + kDispThreads - 1) / kDispThreads;
   // Rows of the padded space this batch can reach: every expert rounds its
   // rows up to a multiple of 32.
@@ -235,7 +301,8 @@ hipError_t launch_dispatch(const int *topk_i, const int *pos, int T, int E, cons
   const int fill_rows = (int)(reach < d.a_pad_cap ? reach : d.a_pad_cap);
   dispatch_count_kernel<<<n_blk, kDispThreads, 0, s>>>(topk_i, pos, T, E, d.blk_counts, d.rowmap,
                                                        fill_rows, d.perm);
-  dispatch_scan_kernel<<<1, 256, 0, s>>>(d.blk_counts, n_blk, E, d.offsets, d.info, d.totals);
+  dispatch_scan_kernel<<<1, 256, 0, s>>>(d.blk_counts, n_blk, E, n_ct_gate_up, n_ct_down, d.offsets,
+                                         d.info, d.totals);
   dispatch_scatter_kernel<<<n_blk, kDispThreads, 0, s>>>(topk_i, pos, T, E, d.blk_counts, d.offsets,
                                                          d.info, d.perm, d.rowmap, d.inv);
   return hipGetLastError();

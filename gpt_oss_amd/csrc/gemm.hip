@@ -28,9 +28,10 @@
 //
 // Tile order.  Workgroup ids are dealt round-robin to the 8 XCDs, each with
 // its own L2.  Logical tile ids are laid out (expert, column tile, row tile)
-// with the row tile fastest, and XCD x takes the x-th contiguous eighth of
-// them: the tiles an XCD runs at one time share the expert's rows and a few
-// column slabs of its weights, so each weight byte leaves HBM once.
+// with the row tile fastest, and XCD x takes a contiguous range of them (see
+// dispatch_scan_kernel: about an eighth by estimated cost): the tiles an XCD
+// runs at one time share the expert's rows and a few column slabs of its
+// weights, so each weight byte leaves HBM once.
 #include <type_traits>
 
 #include "moe_internal.h"
@@ -82,15 +83,13 @@ struct TileCoord {
 // Maps the workgroup id to a tile (see "Tile order" above).  Returns false for
 // the surplus workgroups of the upper-bound grid.
 __device__ __forceinline__ bool locate_tile(const ExpertInfo *__restrict__ info,
-                                            const int *__restrict__ totals, int E, int n_ct,
+                                            const int *__restrict__ bounds, int E, int n_ct,
                                             TileCoord &tc, int &rb) {
-  const int total = totals[0] * n_ct;
-  const int per_xcd = (total + 7) >> 3;
   const int bid = blockIdx.x;
-  const int idx = bid >> 3;
-  if (idx >= per_xcd) return false;
-  const int L = (bid & 7) * per_xcd + idx;
-  if (L >= total) return false;
+  const int xcd = bid & (kXcds - 1);
+  const int first = bounds[xcd];
+  const int L = first + (bid >> 3);
+  if (L >= bounds[xcd + 1]) return false;
   // largest e with tile_base[e] * n_ct <= L and n_mt[e] > 0
   int lo = 0, hi = E - 1;
   while (lo < hi) {
@@ -98,8 +97,8 @@ __device__ __forceinline__ bool locate_tile(const ExpertInfo *__restrict__ info,
     if (info[mid].tile_base * n_ct <= L) lo = mid; else hi = mid - 1;
   }
   // An expert without rows shares tile_base with its successor, so the search
-  // passes over it; a trailing run of empty experts has tile_base == totals[0]
-  // and cannot be reached because L < total.
+  // passes over it; a trailing run of empty experts has tile_base equal to the
+  // number of row tiles and cannot be reached because L is a valid tile.
   const int e = lo;
   const ExpertInfo inf = info[e];
   const int rem = L - inf.tile_base * n_ct;
@@ -107,8 +106,9 @@ __device__ __forceinline__ bool locate_tile(const ExpertInfo *__restrict__ info,
   tc.e = e;
   tc.nt = rem / inf.n_mt;
   rb = inf.rb + (mt < inf.extra ? 1 : 0);
-  tc.rows0 = (mt * inf.rb + min(mt, inf.extra)) * kRowBlock;
-  tc.rb0 = (inf.row0 + tc.rows0) / kRowBlock;
+  const int rb_first = mt * inf.rb + min(mt, inf.extra);  // relative to the expert's segment
+  tc.rows0 = rb_first * kRowBlock;
+  tc.rb0 = inf.row0 / kRowBlock + rb_first;
   return true;
 }
 
@@ -463,7 +463,7 @@ __global__ __launch_bounds__(C::THREADS) void grouped_gemm_kernel(
   const int n_ct = (nb_total + C::TILE_NB - 1) / C::TILE_NB;
   TileCoord tc;
   int rb;
-  if (!locate_tile(info, totals, E, n_ct, tc, rb)) return;
+  if (!locate_tile(info, totals + (GATE_UP ? kTotBoundsGateUp : kTotBoundsDown), E, n_ct, tc, rb)) return;
   const int nb0 = tc.nt * C::TILE_NB;
   const int nb_valid = min(C::TILE_NB, nb_total - nb0);
   const uint4 *b_frag = w_frag + (size_t)tc.e * nb_total * KB * 64;
@@ -482,7 +482,8 @@ __global__ __launch_bounds__(C::THREADS) void grouped_gemm_kernel(
 // 4 waves, one per SIMD, each 256 rows x 64 columns (8 x 2 accumulators = all
 // 256 accumulation registers); 256 x 256 tiles; 7 ring slots.
 using CfgGemm = GemmCfg<4, 2, 7>;
-static_assert(CfgGemm::RBT_MAX * kRowBlock == kTileRows, "tile plan of dispatch_scan_kernel");
+static_assert(CfgGemm::RBT_MAX * kRowBlock == kTileRows && CfgGemm::TILE_NB == kGemmTileNb,
+              "tile plan of dispatch_scan_kernel");
 
 template <typename C, bool GATE_UP>
 static hipError_t launch_gemm(const uint4 *a, const uint4 *w, const float *ba, const float *bb,
@@ -490,7 +491,7 @@ static hipError_t launch_gemm(const uint4 *a, const uint4 *w, const float *ba, c
                               int mt_cap, hipStream_t s) {
   const int nb_total = (GATE_UP ? 2 * N : N) / kRowBlock;
   const int n_ct = (nb_total + C::TILE_NB - 1) / C::TILE_NB;
-  const int grid = ((mt_cap * n_ct + 7) / 8) * 8;
+  const int grid = kXcds * xcd_tile_cap(mt_cap * n_ct);
   grouped_gemm_kernel<C, GATE_UP><<<grid, C::THREADS, 0, s>>>(a, w, ba, bb, d.info, d.totals, out, K,
                                                               N, E, limit);
   return hipGetLastError();

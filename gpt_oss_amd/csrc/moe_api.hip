@@ -116,6 +116,14 @@ struct StageTimer {
   }
 };
 
+// column tiles of the two grouped GEMMs (tiles are kGemmTileNb blocks of 32 columns wide)
+inline int gate_up_col_tiles(const moe_config &c) {
+  return (2 * c.inter / kRowBlock + kGemmTileNb - 1) / kGemmTileNb;
+}
+inline int down_col_tiles(const moe_config &c) {
+  return (c.hidden / kRowBlock + kGemmTileNb - 1) / kGemmTileNb;
+}
+
 int run_experts(moe_handle *h, int layer, const uint16_t *x, const int *pos, const int *topk_i,
                 const float *topk_v, int T, float *out, int accumulate, hipStream_t s,
                 StageTimer &tm) {
@@ -125,7 +133,7 @@ int run_experts(moe_handle *h, int layer, const uint16_t *x, const int *pos, con
   const int mt_cap = A / kTileRows + c.experts;
   const int rb_cap = (A + kTileGran * c.experts + kRowBlock - 1) / kRowBlock;
   HIP_TRY(tm.mark(MOE_STAGE_DISPATCH));
-  HIP_TRY(launch_dispatch(topk_i, pos, T, c.experts, h->disp, s));
+  HIP_TRY(launch_dispatch(topk_i, pos, T, c.experts, gate_up_col_tiles(c), down_col_tiles(c), h->disp, s));
   HIP_TRY(tm.mark(MOE_STAGE_GATHER));
   HIP_TRY(launch_gather(x, h->disp, h->xg, T, c.hidden, rb_cap, s));
   HIP_TRY(tm.mark(MOE_STAGE_GATE_UP));
@@ -189,7 +197,7 @@ int moe_create(const moe_config *cfg, moe_handle **out) {
   ALLOC(h->disp.rowmap, (size_t)h->a_pad_cap);
   ALLOC(h->disp.inv, (size_t)h->a_cap);
   ALLOC(h->disp.info, (size_t)E);
-  ALLOC(h->disp.totals, (size_t)4);
+  ALLOC(h->disp.totals, (size_t)kTotInts);
   ALLOC(h->xg, (size_t)h->a_pad_cap * H);
   ALLOC(h->act, (size_t)h->a_pad_cap * IM);
   ALLOC(h->y, (size_t)h->a_pad_cap * H);
@@ -303,8 +311,8 @@ int moe_dispatch(moe_handle *h, const int *topk_i, const int *pos, int n_tokens,
   if (n_tokens > h->cfg.max_tokens)
     return fail(MOE_ERR_CAPACITY, "n_tokens %d exceeds max_tokens %d", n_tokens, h->cfg.max_tokens);
   if (n_tokens > 0 && !topk_i) return fail(MOE_ERR_BAD_ARG, "null device pointer");
-  HIP_TRY(launch_dispatch(topk_i, pos, n_tokens, h->cfg.experts, h->disp,
-                          static_cast<hipStream_t>(stream)));
+  HIP_TRY(launch_dispatch(topk_i, pos, n_tokens, h->cfg.experts, gate_up_col_tiles(h->cfg),
+                          down_col_tiles(h->cfg), h->disp, static_cast<hipStream_t>(stream)));
   return MOE_OK;
 }
 

@@ -17,6 +17,30 @@ constexpr int kTileRows = 256;  // tallest row tile of the grouped GEMMs
 constexpr int kTileGran = 32;   // an expert's segment of padded rows is a multiple of one row block
 constexpr float kAlpha = 1.702f;  // run.cpp:709
 
+// Work split of the grouped GEMMs over the 8 XCDs (each has an L2 of its own).
+// Tiles are numbered (expert, column tile, row tile), row tile fastest; XCD x
+// takes the tiles [bounds[x], bounds[x+1]), a range of about an eighth of the
+// estimated cost.  (Cutting the last tiles of a range into smaller pieces, so
+// that its CUs run dry together, was measured and does not pay: the pieces are
+// less efficient than what they save.)
+constexpr int kGemmTileNb = 8;  // column blocks (of 32) per tile of the grouped GEMMs
+constexpr int kXcds = 8;
+// estimated cost of a tile: kCostPerTile + kCostPerRowBlock * row blocks.  The
+// fixed part (4 row blocks' worth) was fitted on measured runs with even,
+// Zipf-skewed and 128-expert routing; it stands for the column operand, which
+// a tile streams in full however few rows it has.
+constexpr int kCostPerTile = 32;
+constexpr int kCostPerRowBlock = 8;
+// layout of DispatchBuffers::totals
+constexpr int kTotTiles = 0, kTotRows = 1, kTotAssign = 2;
+constexpr int kTotBoundsGateUp = 4;            // 9 ints
+constexpr int kTotBoundsDown = 4 + kXcds + 1;  // 9 ints
+constexpr int kTotInts = 4 + 2 * (kXcds + 1);
+
+// Most tiles one XCD can be given out of `total`: the balancing never moves a
+// boundary further than this, so that the launch grid can be sized on the host.
+__host__ __device__ inline int xcd_tile_cap(int total) { return (total + 7) / 8 + (total + 15) / 16 + 1; }
+
 // Per-expert record written by the scan kernel and read by the GEMMs.
 struct ExpertInfo {
   int row0;       // first padded row of the expert's segment (multiple of 32)
@@ -59,11 +83,11 @@ struct DispatchBuffers {
   int *rowmap;        // [A_pad] padded position -> assignment id, -1 = padding
   int *inv;           // [A]     assignment id -> padded position, -1 = inactive
   ExpertInfo *info;   // [E]
-  int *totals;        // [4]: total row tiles, total padded rows, total assignments
+  int *totals;        // [kTotInts]: total row tiles, padded rows, assignments; XCD bounds of both GEMMs
   int a_pad_cap;      // capacity of rowmap in rows
 };
-hipError_t launch_dispatch(const int *topk_i, const int *pos, int T, int E, const DispatchBuffers &d,
-                           hipStream_t s);
+hipError_t launch_dispatch(const int *topk_i, const int *pos, int T, int E, int n_ct_gate_up,
+                           int n_ct_down, const DispatchBuffers &d, hipStream_t s);
 hipError_t launch_gather(const uint16_t *x, const DispatchBuffers &d, uint16_t *xg, int T, int H,
                          int rb_cap, hipStream_t s);
 
