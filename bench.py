@@ -28,7 +28,7 @@ PEAK_HBM_GBS = 8000.0
 # HBM bytes per gate_up launch at the c2 workload from rocprofv3 --pmc
 # (FETCH_SIZE + WRITE_SIZE, scaled by the same counters on a copy kernel);
 # None until measured for the workload being run.
-MEASURED_TRAFFIC_BYTES = {"c2": 1.564e9}  # profiles/bench_c2_counters.md
+MEASURED_TRAFFIC_BYTES = {"c2": 1.552e9}  # profiles/bench_c2_counters.md
 
 
 def cpu_baseline(shape, L, budget_s=15.0):
