@@ -19,7 +19,8 @@ STAGES = ["router", "dispatch", "gather", "gate_up", "down", "combine"]
 
 # every symbol include/moe_abi.h declares
 SYMBOLS = [
-    "moe_create", "moe_destroy", "moe_upload_layer", "moe_forward", "moe_router",
+    "moe_create", "moe_destroy", "moe_upload_layer", "moe_upload_layer_mxfp4", "moe_forward",
+    "moe_router",
     "moe_dispatch", "moe_get_dispatch", "moe_experts", "moe_profile_enable",
     "moe_profile_read", "moe_weight_bytes", "moe_workspace_bytes", "moe_last_error",
     "moe_version", "moe_dev_alloc", "moe_dev_free", "moe_dev_upload", "moe_dev_download",
@@ -53,6 +54,7 @@ def lib() -> C.CDLL:
         L.moe_create.argtypes = [C.POINTER(MoeConfig), C.POINTER(vp)]
         L.moe_destroy.argtypes = [vp]
         L.moe_upload_layer.argtypes = [vp, ci] + [vp] * 6
+        L.moe_upload_layer_mxfp4.argtypes = [vp, ci] + [vp] * 8
         L.moe_forward.argtypes = [vp, ci, vp, vp, ci, vp, ci, vp]
         L.moe_router.argtypes = [vp, ci, vp, vp, ci, vp, vp, vp, vp]
         L.moe_dispatch.argtypes = [vp, vp, vp, ci, vp]
@@ -161,6 +163,15 @@ class Moe:
         arrs = [np.ascontiguousarray(a, dtype=np.float32)
                 for a in (w_router, b_router, w_mlp1, b_mlp1, w_mlp2, b_mlp2)]
         check(lib().moe_upload_layer(self.h, layer, *[a.ctypes.data for a in arrs]))
+
+    def upload_layer_mxfp4(self, layer, w_router, b_router, w1_blocks, w1_scales, b_mlp1,
+                           w2_blocks, w2_scales, b_mlp2):
+        """Expert matrices as MXFP4: blocks u8 [E, rows, cols/32, 16], scales u8 [E, rows, cols/32]."""
+        f = lambda a: np.ascontiguousarray(a, dtype=np.float32)
+        u = lambda a: np.ascontiguousarray(a, dtype=np.uint8)
+        arrs = [f(w_router), f(b_router), u(w1_blocks), u(w1_scales), f(b_mlp1), u(w2_blocks),
+                u(w2_scales), f(b_mlp2)]
+        check(lib().moe_upload_layer_mxfp4(self.h, layer, *[a.ctypes.data for a in arrs]))
 
     def forward(self, layer, x, pos, n_tokens, out, accumulate=False, stream=None):
         check(lib().moe_forward(self.h, layer, _p(x), _p(pos), n_tokens, _p(out),

@@ -1,4 +1,7 @@
 // Stand-alone measurement tool (not part of the library):
+//   ingest_probe mfma     sustained rate of v_mfma_f32_32x32x16_bf16 from registers
+//                         alone, and the shader clock it runs at, for 64 / 128 /
+//                         256 busy CUs
 //   ingest_probe stream   per-CU streaming rate L2/MALL/HBM -> LDS (DMA) and -> VGPR
 //   ingest_probe copy N   one plain copy kernel of N MiB, for calibrating the
 //                         FETCH_SIZE / WRITE_SIZE counters of rocprofv3 --pmc
@@ -89,7 +92,72 @@ __global__ void copy_kernel(const uint4 *src, uint4 *dst, size_t n) {
     dst[i] = src[i];
 }
 
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float f32x16_t __attribute__((ext_vector_type(16)));
+
+// 4 waves per workgroup, one per SIMD; 16 independent accumulators per wave, no
+// memory traffic.  out[2*wg] = shader clocks (s_memtime), out[2*wg+1] = 100 MHz
+// ticks (s_memrealtime) spent in the loop.
+__global__ __launch_bounds__(256) void mfma_kernel(int iters, unsigned long long *out, float *sink) {
+  f32x16_t acc[16];
+#pragma unroll
+  for (int i = 0; i < 16; i++)
+#pragma unroll
+    for (int q = 0; q < 16; q++) acc[i][q] = 0.f;
+  bf16x8_t a, b;
+#pragma unroll
+  for (int j = 0; j < 8; j++) {
+    a[j] = (__bf16)(0.001f * (float)(threadIdx.x + j));
+    b[j] = (__bf16)(0.002f * (float)(threadIdx.x ^ j));
+  }
+  const unsigned long long c0 = clock64(), t0 = wall_clock64();
+  for (int it = 0; it < iters; it++) {
+#pragma unroll
+    for (int i = 0; i < 16; i++) acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, acc[i], 0, 0, 0);
+  }
+  const unsigned long long c1 = clock64(), t1 = wall_clock64();
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < 16; i++) s += acc[i][0];
+  if (s == 123.456f) sink[0] = s;
+  if (threadIdx.x == 0) {
+    out[2 * blockIdx.x] = c1 - c0;
+    out[2 * blockIdx.x + 1] = t1 - t0;
+  }
+}
+
+static void run_mfma(int grid) {
+  const int iters = 20000;  // x 16 MFMAs of 32 clocks: about 5 ms
+  unsigned long long *out, host[2 * 256];
+  float *sink;
+  CK(hipMalloc(&out, sizeof host));
+  CK(hipMalloc(&sink, 4));
+  hipEvent_t e0, e1;
+  CK(hipEventCreate(&e0));
+  CK(hipEventCreate(&e1));
+  mfma_kernel<<<grid, 256>>>(1000, out, sink);
+  CK(hipDeviceSynchronize());
+  CK(hipEventRecord(e0));
+  mfma_kernel<<<grid, 256>>>(iters, out, sink);
+  CK(hipEventRecord(e1));
+  CK(hipDeviceSynchronize());
+  float ms;
+  CK(hipEventElapsedTime(&ms, e0, e1));
+  CK(hipMemcpy(host, out, sizeof(unsigned long long) * 2 * grid, hipMemcpyDeviceToHost));
+  double clk = 0, ticks = 0;
+  for (int i = 0; i < grid; i++) { clk += (double)host[2 * i]; ticks += (double)host[2 * i + 1]; }
+  const double flop = (double)grid * 4 * iters * 16 * 2.0 * 32 * 32 * 16;
+  printf("%3d workgroups (one per CU): %7.1f TFLOP/s, shader clock %.2f GHz, %.1f clocks per MFMA per SIMD\n",
+         grid, flop / (ms * 1e-3) / 1e12, clk / (ticks * 10.0), clk / grid / ((double)iters * 16));
+  CK(hipFree(out));
+  CK(hipFree(sink));
+}
+
 int main(int argc, char **argv) {
+  if (argc >= 2 && !strcmp(argv[1], "mfma")) {
+    for (int grid : {64, 128, 256}) run_mfma(grid);
+    return 0;
+  }
   if (argc >= 3 && !strcmp(argv[1], "copy")) {
     const size_t bytes = (size_t)atol(argv[2]) << 20;
     uint4 *a, *b;

@@ -229,14 +229,18 @@ int moe_destroy(moe_handle *h) {
   return MOE_OK;
 }
 
-int moe_upload_layer(moe_handle *h, int layer, const float *w_router, const float *b_router,
-                     const float *w_mlp1, const float *b_mlp1, const float *w_mlp2,
-                     const float *b_mlp2) {
-  if (!h) return fail(MOE_ERR_BAD_ARG, "null handle");
-  if (layer < 0 || layer >= h->cfg.layers)
-    return fail(MOE_ERR_BAD_ARG, "layer %d out of range [0,%d)", layer, h->cfg.layers);
-  if (!w_router || !b_router || !w_mlp1 || !b_mlp1 || !w_mlp2 || !b_mlp2)
-    return fail(MOE_ERR_BAD_ARG, "null weight pointer");
+namespace {
+
+// Source of one layer's expert matrices: fp32 as the reference keeps them on
+// the host, or MXFP4 blocks and scales as the checkpoints hold them.
+struct ExpertSource {
+  const float *w1 = nullptr, *w2 = nullptr;
+  const uint8_t *w1_blocks = nullptr, *w1_scales = nullptr, *w2_blocks = nullptr, *w2_scales = nullptr;
+  bool mxfp4 = false;
+};
+
+int upload_layer(moe_handle *h, int layer, const float *w_router, const float *b_router,
+                 const float *b_mlp1, const float *b_mlp2, const ExpertSource &src) {
   const int E = h->cfg.experts, H = h->cfg.hidden, IM = h->cfg.inter, E_pad = h->E_pad;
   LayerWeights &lw = h->layers[layer];
   int rc = MOE_OK;
@@ -252,8 +256,8 @@ int moe_upload_layer(moe_handle *h, int layer, const float *w_router, const floa
 #undef ALLOCW
   if (rc != MOE_OK) return rc;
 
-  // fp32 staging for one expert matrix at a time; conversion and re-ordering
-  // run on the GPU (the reference packs on the host, utility.cpp:568-622).
+  // Staging for one expert matrix at a time; conversion and re-ordering run on
+  // the GPU (the reference packs on the host, utility.cpp:568-622).
   const size_t stage_elems = (size_t)2 * IM * H > (size_t)E * H ? (size_t)2 * IM * H : (size_t)E * H;
   float *stage = nullptr, *stage_b = nullptr;
   HIP_TRY(hipMalloc(reinterpret_cast<void **>(&stage), stage_elems * sizeof(float)));
@@ -274,15 +278,32 @@ int moe_upload_layer(moe_handle *h, int layer, const float *w_router, const floa
     HIP_TRY(hipMemcpy(stage_b, b_mlp2, (size_t)E * H * sizeof(float), hipMemcpyHostToDevice));
     HIP_TRY(launch_pack_bias(stage_b, lw.b2, nullptr, E * H, false, nullptr));
     HIP_TRY(hipDeviceSynchronize());
+    // the staging buffer holds either an fp32 matrix or, in its place, the
+    // (eight times smaller) blocks followed by the scales of an MXFP4 matrix
+    uint8_t *stage_u8 = reinterpret_cast<uint8_t *>(stage);
+    const size_t n1 = (size_t)2 * IM * H, n2 = (size_t)H * IM;
     for (int ex = 0; ex < E; ex++) {
-      HIP_TRY(hipMemcpy(stage, w_mlp1 + (size_t)ex * 2 * IM * H, (size_t)2 * IM * H * sizeof(float),
-                        hipMemcpyHostToDevice));
-      HIP_TRY(launch_pack_weight(stage, lw.w1 + (size_t)ex * 2 * IM * H, 2 * IM, H, true, nullptr));
-      HIP_TRY(hipDeviceSynchronize());
-      HIP_TRY(hipMemcpy(stage, w_mlp2 + (size_t)ex * H * IM, (size_t)H * IM * sizeof(float),
-                        hipMemcpyHostToDevice));
-      HIP_TRY(launch_pack_weight(stage, lw.w2 + (size_t)ex * H * IM, H, IM, false, nullptr));
-      HIP_TRY(hipDeviceSynchronize());
+      if (!src.mxfp4) {
+        HIP_TRY(hipMemcpy(stage, src.w1 + ex * n1, n1 * sizeof(float), hipMemcpyHostToDevice));
+        HIP_TRY(launch_pack_weight(stage, lw.w1 + ex * n1, 2 * IM, H, true, nullptr));
+        HIP_TRY(hipDeviceSynchronize());
+        HIP_TRY(hipMemcpy(stage, src.w2 + ex * n2, n2 * sizeof(float), hipMemcpyHostToDevice));
+        HIP_TRY(launch_pack_weight(stage, lw.w2 + ex * n2, H, IM, false, nullptr));
+        HIP_TRY(hipDeviceSynchronize());
+      } else {
+        HIP_TRY(hipMemcpy(stage_u8, src.w1_blocks + ex * (n1 / 2), n1 / 2, hipMemcpyHostToDevice));
+        HIP_TRY(hipMemcpy(stage_u8 + n1 / 2, src.w1_scales + ex * (n1 / 32), n1 / 32,
+                          hipMemcpyHostToDevice));
+        HIP_TRY(launch_pack_weight_mxfp4(stage_u8, stage_u8 + n1 / 2, lw.w1 + ex * n1, 2 * IM, H, true,
+                                         nullptr));
+        HIP_TRY(hipDeviceSynchronize());
+        HIP_TRY(hipMemcpy(stage_u8, src.w2_blocks + ex * (n2 / 2), n2 / 2, hipMemcpyHostToDevice));
+        HIP_TRY(hipMemcpy(stage_u8 + n2 / 2, src.w2_scales + ex * (n2 / 32), n2 / 32,
+                          hipMemcpyHostToDevice));
+        HIP_TRY(launch_pack_weight_mxfp4(stage_u8, stage_u8 + n2 / 2, lw.w2 + ex * n2, H, IM, false,
+                                         nullptr));
+        HIP_TRY(hipDeviceSynchronize());
+      }
     }
     return MOE_OK;
   };
@@ -291,6 +312,46 @@ int moe_upload_layer(moe_handle *h, int layer, const float *w_router, const floa
   (void)hipFree(stage_b);
   if (rc == MOE_OK) lw.uploaded = true;
   return rc;
+}
+
+int check_upload_args(moe_handle *h, int layer) {
+  if (!h) return fail(MOE_ERR_BAD_ARG, "null handle");
+  if (layer < 0 || layer >= h->cfg.layers)
+    return fail(MOE_ERR_BAD_ARG, "layer %d out of range [0,%d)", layer, h->cfg.layers);
+  return MOE_OK;
+}
+
+}  // namespace
+
+int moe_upload_layer(moe_handle *h, int layer, const float *w_router, const float *b_router,
+                     const float *w_mlp1, const float *b_mlp1, const float *w_mlp2,
+                     const float *b_mlp2) {
+  const int rc = check_upload_args(h, layer);
+  if (rc != MOE_OK) return rc;
+  if (!w_router || !b_router || !w_mlp1 || !b_mlp1 || !w_mlp2 || !b_mlp2)
+    return fail(MOE_ERR_BAD_ARG, "null weight pointer");
+  ExpertSource src;
+  src.w1 = w_mlp1;
+  src.w2 = w_mlp2;
+  return upload_layer(h, layer, w_router, b_router, b_mlp1, b_mlp2, src);
+}
+
+int moe_upload_layer_mxfp4(moe_handle *h, int layer, const float *w_router, const float *b_router,
+                           const uint8_t *w_mlp1_blocks, const uint8_t *w_mlp1_scales,
+                           const float *b_mlp1, const uint8_t *w_mlp2_blocks,
+                           const uint8_t *w_mlp2_scales, const float *b_mlp2) {
+  const int rc = check_upload_args(h, layer);
+  if (rc != MOE_OK) return rc;
+  if (!w_router || !b_router || !w_mlp1_blocks || !w_mlp1_scales || !b_mlp1 || !w_mlp2_blocks ||
+      !w_mlp2_scales || !b_mlp2)
+    return fail(MOE_ERR_BAD_ARG, "null weight pointer");
+  ExpertSource src;
+  src.mxfp4 = true;
+  src.w1_blocks = w_mlp1_blocks;
+  src.w1_scales = w_mlp1_scales;
+  src.w2_blocks = w_mlp2_blocks;
+  src.w2_scales = w_mlp2_scales;
+  return upload_layer(h, layer, w_router, b_router, b_mlp1, b_mlp2, src);
 }
 
 int moe_router(moe_handle *h, int layer, const uint16_t *x, const int *pos, int n_tokens,

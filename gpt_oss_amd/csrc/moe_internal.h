@@ -69,6 +69,8 @@ hipError_t launch_pack_router(const float *w_src, const float *b_src, uint16_t *
                               int E, int E_pad, int H, hipStream_t s);
 hipError_t launch_pack_weight(const float *src, uint16_t *dst, int rows, int cols, bool gate_up,
                               hipStream_t s);
+hipError_t launch_pack_weight_mxfp4(const uint8_t *blocks, const uint8_t *scales, uint16_t *dst,
+                                    int rows, int cols, bool gate_up, hipStream_t s);
 hipError_t launch_pack_bias(const float *src, float *dst_a, float *dst_b, int n, bool deinterleave,
                             hipStream_t s);
 

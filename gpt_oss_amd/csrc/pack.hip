@@ -52,6 +52,47 @@ __global__ void pack_weight_kernel(const float *__restrict__ src, uint4 *__restr
   }
 }
 
+// MXFP4 ingest (export_model_bin/gpt-oss-20b/export_model_bin.py:86-123): a
+// row of `cols` weights is cols/32 blocks of 16 bytes plus one scale byte per
+// block; byte b of a block holds element 2b in its low nibble and element 2b+1
+// in its high nibble; a nibble indexes the table below and the scale byte s
+// multiplies by 2^(s - 127) (ldexp, as the exporter does).  Output: the same
+// bf16 fragments as pack_weight_kernel writes, so the GEMMs do not know the
+// difference.  The table values carry two significant bits, so the bf16 result
+// is exact wherever it is in range.
+__constant__ float kFp4Values[16] = {+0.0f, +0.5f, +1.0f, +1.5f, +2.0f, +3.0f, +4.0f, +6.0f,
+                                     -0.0f, -0.5f, -1.0f, -1.5f, -2.0f, -3.0f, -4.0f, -6.0f};
+
+__global__ void pack_weight_mxfp4_kernel(const uint8_t *__restrict__ blocks,
+                                         const uint8_t *__restrict__ scales, uint4 *__restrict__ dst,
+                                         int rows, int cols, int gate_up) {
+  const int kb_total = cols / kFragK;
+  const int groups = cols / 32;
+  const size_t n_chunks = (size_t)(rows / kRowBlock) * kb_total * 64;
+  for (size_t c = (size_t)blockIdx.x * blockDim.x + threadIdx.x; c < n_chunks;
+       c += (size_t)gridDim.x * blockDim.x) {
+    const int lane = (int)(c & 63);
+    const size_t frag = c >> 6;
+    const int kb = (int)(frag % kb_total);
+    const int nb = (int)(frag / kb_total);
+    const int n = lane & 31;
+    const int k0 = kb * kFragK + 8 * (lane >> 5);  // 8 consecutive elements of one block
+    const int row = gate_up ? 2 * (kRowBlock * (nb >> 1) + n) + (nb & 1) : kRowBlock * nb + n;
+    const size_t g = (size_t)row * groups + k0 / 32;
+    const uint32_t bytes = *reinterpret_cast<const uint32_t *>(blocks + g * 16 + (k0 % 32) / 2);
+    const int expo = (int)scales[g] - 127;
+    uint32_t o[4];
+#pragma unroll
+    for (int b = 0; b < 4; b++) {
+      const uint32_t byte = (bytes >> (8 * b)) & 0xffu;
+      const float lo = ldexpf(kFp4Values[byte & 15u], expo);
+      const float hi = ldexpf(kFp4Values[byte >> 4], expo);
+      o[b] = f32_to_bf16_rne(lo) | ((uint32_t)f32_to_bf16_rne(hi) << 16);
+    }
+    dst[c] = make_uint4(o[0], o[1], o[2], o[3]);
+  }
+}
+
 // Router weight in the operand order of v_mfma_f64_16x16x4_f64, kept as bf16
 // (the kernel widens to f64 on the fly: a quarter of the bytes of an f64 copy,
 // and the router is otherwise bound by streaming this matrix through every CU).
@@ -103,6 +144,13 @@ hipError_t launch_pack_weight(const float *src, uint16_t *dst, int rows, int col
                               hipStream_t s) {
   pack_weight_kernel<<<2048, 256, 0, s>>>(src, reinterpret_cast<uint4 *>(dst), rows, cols,
                                           gate_up ? 1 : 0);
+  return hipGetLastError();
+}
+
+hipError_t launch_pack_weight_mxfp4(const uint8_t *blocks, const uint8_t *scales, uint16_t *dst,
+                                    int rows, int cols, bool gate_up, hipStream_t s) {
+  pack_weight_mxfp4_kernel<<<2048, 256, 0, s>>>(blocks, scales, reinterpret_cast<uint4 *>(dst), rows,
+                                                cols, gate_up ? 1 : 0);
   return hipGetLastError();
 }
 

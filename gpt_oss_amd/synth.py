@@ -42,6 +42,8 @@ CONFIGS = {
     "c3b": LayerShape("c3b", 7168, 2880, 2880, 32, zipf=1.2),
     # GPT-OSS-120B shape
     "c4": LayerShape("c4", 6144, 2880, 2880, 128),
+    # 20B shape, expert matrices given as MXFP4 blocks and scales (make_experts_mxfp4)
+    "c5": LayerShape("c5", 64, 2880, 2880, 32),
 }
 
 
@@ -141,6 +143,22 @@ def make_experts(shape: LayerShape, seed: int = 0):
     w2 = _normal(seed, 6, (E, H, IM), 0.02, shape.bf16)
     b2 = _normal(seed, 7, (E, H), 0.02, shape.bf16)
     return w1, b1, w2, b2
+
+
+def make_experts_mxfp4(shape: LayerShape, seed: int = 0):
+    """MXFP4 expert matrices: per 32 weights 16 random bytes (uniform nibbles) and
+    a scale byte uniform in [119, 129] (exponents -8 .. 2); biases as make_experts.
+    Returns (w1_blocks, w1_scales, b1, w2_blocks, w2_scales, b2) with blocks
+    u8 [E, rows, cols/32, 16] and scales u8 [E, rows, cols/32]."""
+    E, H, IM = shape.experts, shape.hidden, shape.inter
+    rng = np.random.Generator(np.random.PCG64([seed, 40]))
+    w1_blocks = rng.integers(0, 256, (E, 2 * IM, H // 32, 16), dtype=np.uint8)
+    w1_scales = rng.integers(119, 130, (E, 2 * IM, H // 32), dtype=np.uint8)
+    w2_blocks = rng.integers(0, 256, (E, H, IM // 32, 16), dtype=np.uint8)
+    w2_scales = rng.integers(119, 130, (E, H, IM // 32), dtype=np.uint8)
+    b1 = _normal(seed, 5, (E, 2 * IM), 0.02, shape.bf16)
+    b2 = _normal(seed, 7, (E, H), 0.02, shape.bf16)
+    return w1_blocks, w1_scales, b1, w2_blocks, w2_scales, b2
 
 
 def make_layer(shape: LayerShape, seed: int = 0, tokens: int | None = None) -> dict:

@@ -85,6 +85,23 @@ int moe_upload_layer(moe_handle *h, int layer, const float *w_router,
                      const float *b_mlp1, const float *w_mlp2,
                      const float *b_mlp2);
 
+/* As moe_upload_layer, with the expert matrices in MXFP4 as the GPT-OSS
+ * checkpoints hold them: for a matrix [rows, cols] (cols a multiple of 32)
+ * blocks is u8 [E, rows, cols/32, 16] and scales u8 [E, rows, cols/32]; byte b
+ * of a block holds element 2b in its low and element 2b+1 in its high nibble, a
+ * nibble indexes {0, .5, 1, 1.5, 2, 3, 4, 6, -0, -.5, -1, -1.5, -2, -3, -4, -6}
+ * and the scale byte s multiplies by 2^(s-127).  Takes the place of
+ * dequantize_fp4 in the exporter
+ * (export_model_bin/gpt-oss-20b/export_model_bin.py:66-123) followed by the fp32
+ * upload; the decoded values are kept as bf16, which holds them exactly.
+ * Router weights and all biases stay fp32 arguments.  Synchronous. */
+int moe_upload_layer_mxfp4(moe_handle *h, int layer, const float *w_router,
+                           const float *b_router,
+                           const uint8_t *w_mlp1_blocks,
+                           const uint8_t *w_mlp1_scales, const float *b_mlp1,
+                           const uint8_t *w_mlp2_blocks,
+                           const uint8_t *w_mlp2_scales, const float *b_mlp2);
+
 /* The whole layer for one batch: out[t,:] (+)= sum_k w[t,k] * expert_k(x[t,:]).
  *   x    bf16 [n_tokens, H] row-major (the reference's d_t)
  *   pos  int  [n_tokens] or NULL; pos[t] < 0 marks an inactive row, which takes

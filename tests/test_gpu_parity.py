@@ -253,6 +253,42 @@ def test_c4_120b_shape():
     check_outputs(R, L, L["x"], None, rows)
 
 
+def test_c5_mxfp4_ingest():
+    """Expert matrices uploaded as MXFP4 blocks and scales.  The oracle decodes
+    them on the CPU (closed form pinned in tests/test_oracle.py); its values are
+    exact in bf16, so the GPU decode must lead to bit-identical outputs as an
+    upload of the decoded fp32 matrices, and the layer must match the oracle run
+    on those matrices.  Outputs are large here (weights up to 24), hence the
+    absolute bar scales with the output."""
+    sh = synth.CONFIGS["c5"]
+    x = synth.round_bf16(synth.make_activations(sh))
+    wr, br = (synth.round_bf16(a) for a in synth.make_router(sh))
+    b1k, s1, b1, b2k, s2, b2 = synth.make_experts_mxfp4(sh)
+    b1, b2 = synth.round_bf16(b1), synth.round_bf16(b2)
+    w1 = ob.mxfp4_dequant(b1k, s1)
+    w2 = ob.mxfp4_dequant(b2k, s2)
+    assert w1.shape == (sh.experts, 2 * sh.inter, sh.hidden) and np.array_equal(w1, synth.round_bf16(w1))
+    L = dict(w_router=wr, b_router=br, w_mlp1=w1, b_mlp1=b1, w_mlp2=w2, b_mlp2=b2)
+
+    m4 = abi.Moe(sh.hidden, sh.inter, sh.experts, max_tokens=sh.tokens, swiglu_limit=sh.limit)
+    m4.upload_layer_mxfp4(0, wr, br, b1k, s1, b1, b2k, s2, b2)
+    R4 = abi.run_layer(m4, 0, x, None)
+    m32 = make_moe(sh, L, sh.tokens)
+    R32 = abi.run_layer(m32, 0, x, None)
+    assert np.array_equal(R4["topk_i"], R32["topk_i"])
+    assert np.array_equal(R4["out"], R32["out"]), "MXFP4 decode on the GPU differs from the oracle's"
+
+    check_routing(R4, L, x, None, sh.experts)
+    rows = np.arange(16)
+    want = oracle_rows(L, x, None, rows)
+    got = R4["out"][rows]
+    assert rel_l2(got, want) <= REL_L2
+    assert np.abs(got - want).max() <= MAX_ABS * max(1.0, float(np.abs(want).max()))
+
+    with pytest.raises(abi.MoeError):
+        m4.upload_layer_mxfp4(3, wr, br, b1k, s1, b1, b2k, s2, b2)  # layer out of range
+
+
 # ---------------- host logic on the GPU box ----------------
 
 def test_error_paths_and_profiling(c2):
