@@ -19,7 +19,8 @@ STAGES = ["router", "dispatch", "gather", "gate_up", "down", "combine"]
 
 # every symbol include/moe_abi.h declares
 SYMBOLS = [
-    "moe_create", "moe_destroy", "moe_upload_layer", "moe_upload_layer_mxfp4", "moe_forward",
+    "moe_create", "moe_destroy", "moe_upload_layer", "moe_upload_layer_mxfp4", "moe_upload_norm",
+    "moe_forward", "moe_block_forward",
     "moe_router",
     "moe_dispatch", "moe_get_dispatch", "moe_experts", "moe_profile_enable",
     "moe_profile_read", "moe_weight_bytes", "moe_workspace_bytes", "moe_last_error",
@@ -56,6 +57,8 @@ def lib() -> C.CDLL:
         L.moe_upload_layer.argtypes = [vp, ci] + [vp] * 6
         L.moe_upload_layer_mxfp4.argtypes = [vp, ci] + [vp] * 8
         L.moe_forward.argtypes = [vp, ci, vp, vp, ci, vp, ci, vp]
+        L.moe_upload_norm.argtypes = [vp, ci, vp]
+        L.moe_block_forward.argtypes = [vp, ci, vp, vp, ci, vp]
         L.moe_router.argtypes = [vp, ci, vp, vp, ci, vp, vp, vp, vp]
         L.moe_dispatch.argtypes = [vp, vp, vp, ci, vp]
         L.moe_get_dispatch.argtypes = [vp, vp, vp, ci, vp]
@@ -172,6 +175,14 @@ class Moe:
         arrs = [f(w_router), f(b_router), u(w1_blocks), u(w1_scales), f(b_mlp1), u(w2_blocks),
                 u(w2_scales), f(b_mlp2)]
         check(lib().moe_upload_layer_mxfp4(self.h, layer, *[a.ctypes.data for a in arrs]))
+
+    def upload_norm(self, layer, rms_w):
+        a = np.ascontiguousarray(rms_w, dtype=np.float32)
+        check(lib().moe_upload_norm(self.h, layer, a.ctypes.data))
+
+    def block_forward(self, layer, x, pos, n_tokens, stream=None):
+        """x: DevBuf of bf16 [n_tokens, H], updated in place."""
+        check(lib().moe_block_forward(self.h, layer, _p(x), _p(pos), n_tokens, stream))
 
     def forward(self, layer, x, pos, n_tokens, out, accumulate=False, stream=None):
         check(lib().moe_forward(self.h, layer, _p(x), _p(pos), n_tokens, _p(out),

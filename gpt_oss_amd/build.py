@@ -9,7 +9,7 @@ PKG = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(PKG, "csrc")
 LIB = os.path.join(PKG, "libmi355_moe.so")
 PROBE = os.path.join(PKG, "ingest_probe.exe")
-SOURCES = ["moe_api.hip", "pack.hip", "router.hip", "dispatch.hip", "gemm.hip"]
+SOURCES = ["moe_api.hip", "pack.hip", "router.hip", "dispatch.hip", "gemm.hip", "norm.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",

@@ -11,6 +11,16 @@ namespace moe {
 
 constexpr int kDispThreads = 256;  // tokens per workgroup in count / scatter
 
+__device__ __forceinline__ uint16_t f32_to_bf16_rne_disp(float f) {
+  uint32_t u = __float_as_uint(f);
+  if (~u & 0x7f800000u) {
+    u += 0x7fffu + ((u >> 16) & 1u);
+  } else if (u & 0xffffu) {
+    u |= 0x10000u;
+  }
+  return (uint16_t)(u >> 16);
+}
+
 // Pass 1: per-workgroup histogram of expert ids over active rows.  Also resets
 // rowmap and perm to -1 (a fill kernel rather than a memset so that the call
 // sequence can be captured in a graph).
@@ -261,14 +271,20 @@ __global__ __launch_bounds__(256) void gather_rows_kernel(const uint16_t *__rest
 // (descending router score, as reduce_mlp2_slots_kernel does,
 // utility/utility.cpp:701-726).  Every token owns its K rows of y, so there
 // are no atomics.
+//
+// RESID: instead of writing the fp32 sum, adds it to the bf16 residual stream
+// in place, x = bf16(float(x) + sum) (residual_add_batch_kernel,
+// utility/utility.cpp:158-173; call getp_run.cpp:846-852); inactive rows are
+// left alone.
+template <bool RESID>
 __global__ __launch_bounds__(256) void combine_kernel(const float *__restrict__ y,
                                                      const int *__restrict__ inv,
                                                      const float *__restrict__ topk_v,
-                                                     const int *__restrict__ pos,
-                                                     float *__restrict__ out, int H, int accumulate) {
+                                                     const int *__restrict__ pos, void *outp, int H,
+                                                     int accumulate) {
   const int t = blockIdx.x;
   const bool active = !(pos && pos[t] < 0);
-  if (!active && accumulate) return;
+  if (!active && (accumulate || RESID)) return;
   int p[kTopK] = {-1, -1, -1, -1};
   float w[kTopK] = {0.f, 0.f, 0.f, 0.f};
   if (active) {
@@ -277,9 +293,10 @@ __global__ __launch_bounds__(256) void combine_kernel(const float *__restrict__ 
     p[0] = pi.x; p[1] = pi.y; p[2] = pi.z; p[3] = pi.w;
     w[0] = wv.x; w[1] = wv.y; w[2] = wv.z; w[3] = wv.w;
   }
-  float4 *o = reinterpret_cast<float4 *>(out + (size_t)t * H);
+  float4 *o = reinterpret_cast<float4 *>(reinterpret_cast<float *>(outp) + (size_t)t * H);
+  uint2 *xr = reinterpret_cast<uint2 *>(reinterpret_cast<uint16_t *>(outp) + (size_t)t * H);
   for (int c = threadIdx.x; c < H / 4; c += 256) {
-    float4 s = accumulate ? o[c] : make_float4(0.f, 0.f, 0.f, 0.f);
+    float4 s = (!RESID && accumulate) ? o[c] : make_float4(0.f, 0.f, 0.f, 0.f);
 #pragma unroll
     for (int k = 0; k < kTopK; k++) {
       if (p[k] >= 0) {
@@ -287,7 +304,15 @@ __global__ __launch_bounds__(256) void combine_kernel(const float *__restrict__ 
         s.x += w[k] * v.x; s.y += w[k] * v.y; s.z += w[k] * v.z; s.w += w[k] * v.w;
       }
     }
-    o[c] = s;
+    if (RESID) {
+      const uint2 xv = xr[c];
+      const float r0 = __uint_as_float(xv.x << 16) + s.x, r1 = __uint_as_float(xv.x & 0xffff0000u) + s.y;
+      const float r2 = __uint_as_float(xv.y << 16) + s.z, r3 = __uint_as_float(xv.y & 0xffff0000u) + s.w;
+      xr[c] = make_uint2(f32_to_bf16_rne_disp(r0) | ((uint32_t)f32_to_bf16_rne_disp(r1) << 16),
+                         f32_to_bf16_rne_disp(r2) | ((uint32_t)f32_to_bf16_rne_disp(r3) << 16));
+    } else {
+      o[c] = s;
+    }
   }
 }
 
@@ -319,7 +344,13 @@ hipError_t launch_gather(const uint16_t *x, const DispatchBuffers &d, uint16_t *
 
 hipError_t launch_combine(const float *y, const int *inv, const float *topk_v, const int *pos,
                           float *out, int T, int H, int accumulate, hipStream_t s) {
-  combine_kernel<<<T, 256, 0, s>>>(y, inv, topk_v, pos, out, H, accumulate);
+  combine_kernel<false><<<T, 256, 0, s>>>(y, inv, topk_v, pos, out, H, accumulate);
+  return hipGetLastError();
+}
+
+hipError_t launch_combine_residual(const float *y, const int *inv, const float *topk_v,
+                                   const int *pos, uint16_t *x, int T, int H, hipStream_t s) {
+  combine_kernel<true><<<T, 256, 0, s>>>(y, inv, topk_v, pos, x, H, 0);
   return hipGetLastError();
 }
 

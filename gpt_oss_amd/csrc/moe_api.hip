@@ -63,6 +63,7 @@ struct moe_handle {
   uint16_t *xg = nullptr;   // gathered rows, bf16 fragments
   uint16_t *act = nullptr;  // SwiGLU output, bf16 fragments
   float *y = nullptr;       // down output [a_pad_cap, H]
+  uint16_t *t_norm = nullptr;  // normalised rows of moe_block_forward [max_tokens, H], allocated on first use
 
   // profiling
   std::vector<hipEvent_t> events;  // kMaxProfileCalls * (MOE_NUM_STAGES + 1)
@@ -124,9 +125,10 @@ inline int down_col_tiles(const moe_config &c) {
   return (c.hidden / kRowBlock + kGemmTileNb - 1) / kGemmTileNb;
 }
 
+// out != nullptr: out (+)= layer(x), fp32.  Otherwise resid (bf16, in place) += layer(x).
 int run_experts(moe_handle *h, int layer, const uint16_t *x, const int *pos, const int *topk_i,
                 const float *topk_v, int T, float *out, int accumulate, hipStream_t s,
-                StageTimer &tm) {
+                StageTimer &tm, uint16_t *resid = nullptr) {
   const moe_config &c = h->cfg;
   const LayerWeights &lw = h->layers[layer];
   const int A = T * kTopK;
@@ -142,7 +144,11 @@ int run_experts(moe_handle *h, int layer, const uint16_t *x, const int *pos, con
   HIP_TRY(tm.mark(MOE_STAGE_DOWN));
   HIP_TRY(launch_down(h->act, lw.w2, lw.b2, h->disp, h->y, c.hidden, c.inter, c.experts, mt_cap, s));
   HIP_TRY(tm.mark(MOE_STAGE_COMBINE));
-  HIP_TRY(launch_combine(h->y, h->disp.inv, topk_v, pos, out, T, c.hidden, accumulate, s));
+  if (out) {
+    HIP_TRY(launch_combine(h->y, h->disp.inv, topk_v, pos, out, T, c.hidden, accumulate, s));
+  } else {
+    HIP_TRY(launch_combine_residual(h->y, h->disp.inv, topk_v, pos, resid, T, c.hidden, s));
+  }
   HIP_TRY(tm.mark(MOE_NUM_STAGES));
   return MOE_OK;
 }
@@ -218,12 +224,12 @@ int moe_destroy(moe_handle *h) {
   if (!h) return MOE_OK;
   for (auto &lw : h->layers) {
     (void)hipFree(lw.wr); (void)hipFree(lw.br); (void)hipFree(lw.w1); (void)hipFree(lw.b1g);
-    (void)hipFree(lw.b1u); (void)hipFree(lw.w2); (void)hipFree(lw.b2);
+    (void)hipFree(lw.b1u); (void)hipFree(lw.w2); (void)hipFree(lw.b2); (void)hipFree(lw.rms_w);
   }
   (void)hipFree(h->topk_i); (void)hipFree(h->topk_v);
   (void)hipFree(h->disp.blk_counts); (void)hipFree(h->disp.offsets); (void)hipFree(h->disp.perm);
   (void)hipFree(h->disp.rowmap); (void)hipFree(h->disp.inv); (void)hipFree(h->disp.info); (void)hipFree(h->disp.totals);
-  (void)hipFree(h->xg); (void)hipFree(h->act); (void)hipFree(h->y);
+  (void)hipFree(h->xg); (void)hipFree(h->act); (void)hipFree(h->y); (void)hipFree(h->t_norm);
   for (hipEvent_t ev : h->events) (void)hipEventDestroy(ev);
   delete h;
   return MOE_OK;
@@ -417,6 +423,48 @@ int moe_forward(moe_handle *h, int layer, const uint16_t *x, const int *pos, int
   HIP_TRY(launch_router(x, pos, lw.wr, lw.br, n_tokens, h->cfg.hidden, h->cfg.experts, h->E_pad,
                         nullptr, h->topk_i, h->topk_v, s));
   rc = run_experts(h, layer, x, pos, h->topk_i, h->topk_v, n_tokens, out, accumulate, s, tm);
+  if (rc == MOE_OK) tm.done();
+  return rc;
+}
+
+int moe_upload_norm(moe_handle *h, int layer, const float *rms_ffn_w) {
+  const int rc0 = check_upload_args(h, layer);
+  if (rc0 != MOE_OK) return rc0;
+  if (!rms_ffn_w) return fail(MOE_ERR_BAD_ARG, "null weight pointer");
+  const int H = h->cfg.hidden;
+  LayerWeights &lw = h->layers[layer];
+  int rc = MOE_OK;
+  if (!lw.rms_w) rc = dev_alloc(h, &lw.rms_w, (size_t)H, false);
+  if (rc == MOE_OK && !h->t_norm) rc = dev_alloc(h, &h->t_norm, (size_t)h->cfg.max_tokens * H, true);
+  if (rc != MOE_OK) return rc;
+  float *stage = nullptr;
+  HIP_TRY(hipMalloc(reinterpret_cast<void **>(&stage), (size_t)H * sizeof(float)));
+  auto body = [&]() -> int {
+    HIP_TRY(hipMemcpy(stage, rms_ffn_w, (size_t)H * sizeof(float), hipMemcpyHostToDevice));
+    HIP_TRY(launch_pack_bias(stage, lw.rms_w, nullptr, H, false, nullptr));  // rounds to bf16 values
+    HIP_TRY(hipDeviceSynchronize());
+    return MOE_OK;
+  };
+  rc = body();
+  (void)hipFree(stage);
+  return rc;
+}
+
+int moe_block_forward(moe_handle *h, int layer, uint16_t *x, const int *pos, int n_tokens,
+                      void *stream) {
+  int rc = check_forward_args(h, layer, x, n_tokens, x);
+  if (rc != MOE_OK) return rc;
+  const LayerWeights &lw = h->layers[layer];
+  if (!lw.rms_w)
+    return fail(MOE_ERR_STATE, "layer %d has no norm weight (moe_upload_norm not called)", layer);
+  if (n_tokens == 0) return MOE_OK;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  StageTimer tm(h, s);
+  HIP_TRY(tm.mark(MOE_STAGE_ROUTER));  // the norm is counted with the router stage
+  HIP_TRY(launch_rmsnorm(x, lw.rms_w, pos, h->t_norm, n_tokens, h->cfg.hidden, s));
+  HIP_TRY(launch_router(h->t_norm, pos, lw.wr, lw.br, n_tokens, h->cfg.hidden, h->cfg.experts,
+                        h->E_pad, nullptr, h->topk_i, h->topk_v, s));
+  rc = run_experts(h, layer, h->t_norm, pos, h->topk_i, h->topk_v, n_tokens, nullptr, 0, s, tm, x);
   if (rc == MOE_OK) tm.done();
   return rc;
 }

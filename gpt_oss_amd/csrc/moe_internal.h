@@ -60,6 +60,7 @@ struct LayerWeights {
   float *b1u = nullptr;    // up bias   [E, IM]
   uint16_t *w2 = nullptr;  // down weight, bf16 MFMA fragments
   float *b2 = nullptr;     // down bias [E, H]
+  float *rms_w = nullptr;  // weight of the RMS norm in front of the layer [H] (bf16 values), optional
   bool uploaded = false;
 };
 
@@ -101,5 +102,9 @@ hipError_t launch_down(const uint16_t *act, const uint16_t *w2, const float *b2,
                        hipStream_t s);
 hipError_t launch_combine(const float *y, const int *inv, const float *topk_v, const int *pos,
                           float *out, int T, int H, int accumulate, hipStream_t s);
+hipError_t launch_combine_residual(const float *y, const int *inv, const float *topk_v,
+                                   const int *pos, uint16_t *x, int T, int H, hipStream_t s);
+hipError_t launch_rmsnorm(const uint16_t *x, const float *weight, const int *pos, uint16_t *t_out,
+                          int T, int H, hipStream_t s);
 
 }  // namespace moe

@@ -14,6 +14,9 @@
 //                          getp_run.cpp:798), no host synchronisation
 //   mi355_moe_forward_fused <- the same plus the router and top-k launches it
 //                          makes redundant (getp_run.cpp:697-716)
+//   mi355_moe_block     <- the whole FFN block of a layer: rmsnorm_batch_kernel, router,
+//                          top-k, local MoE path and residual_add_batch_kernel
+//                          (getp_run.cpp:686-852), in place on d_x
 //   mi355_moe_cleanup   <- cleanup_device_context_ep (expert.cpp:1234-1364)
 // Error behaviour follows HIP_CHECK (common/defines.h:94-102): print and exit.
 #pragma once
@@ -70,6 +73,8 @@ static void mi355_moe_init(DeviceContext &ctx, int device_id, Transformer *trans
         g_mi355_moe[device_id], l, w->w_router + (size_t)l * H * E, w->b_router + (size_t)l * E,
         w->w_mlp1 + (size_t)l * E * 2 * IM * H, w->b_mlp1 + (size_t)l * E * 2 * IM,
         w->w_mlp2 + (size_t)l * E * H * IM, w->b_mlp2 + (size_t)l * E * H));
+    // the reference's device copy is d_rms_ffn_w (getp_run.cpp:161-163)
+    MI355_MOE_CHECK(moe_upload_norm(g_mi355_moe[device_id], l, w->rms_ffn_w + (size_t)l * H));
   }
   (void)ctx;
 }
@@ -95,6 +100,16 @@ static void mi355_moe_forward_fused(DeviceContext &ctx, int batch_size, int laye
                               reinterpret_cast<const uint16_t *>(ctx.gpu_activations.d_t),
                               ctx.gpu_activations.d_pos, batch_size, ctx.gpu_activations.d_e_agg,
                               /*accumulate=*/0, /*stream=*/nullptr));
+}
+
+// The FFN block of one layer in place on the residual stream d_x: replaces
+// getp_run.cpp:686-852 (rmsnorm_batch_kernel into d_t, router, top-k, memset of
+// d_e_agg, local MoE path, residual_add_batch_kernel).  d_t and d_e_agg are not
+// touched.
+static void mi355_moe_block(DeviceContext &ctx, int batch_size, int layer) {
+  MI355_MOE_CHECK(moe_block_forward(mi355_moe_of(ctx), layer,
+                                    reinterpret_cast<uint16_t *>(ctx.gpu_activations.d_x),
+                                    ctx.gpu_activations.d_pos, batch_size, /*stream=*/nullptr));
 }
 
 static void mi355_moe_cleanup(DeviceContext &ctx) {

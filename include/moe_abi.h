@@ -115,6 +115,23 @@ int moe_upload_layer_mxfp4(moe_handle *h, int layer, const float *w_router,
 int moe_forward(moe_handle *h, int layer, const uint16_t *x, const int *pos,
                 int n_tokens, float *out, int accumulate, void *stream);
 
+/* The weight of the RMS norm in front of the layer (rms_ffn_w + layer*H,
+ * run.cpp:51, used at run.cpp:660; device copy d_rms_ffn_w, getp_run.cpp:691),
+ * fp32 [H]; kept as bf16 values like the other weights.  Needed by
+ * moe_block_forward only.  Synchronous. */
+int moe_upload_norm(moe_handle *h, int layer, const float *rms_ffn_w);
+
+/* The FFN block in place on the residual stream x (bf16 [n_tokens, H], the
+ * reference's d_x):  t = rmsnorm(x) * rms_ffn_w;  x = bf16(x + layer(t)).
+ * Replaces rmsnorm_batch_kernel (utility/utility.cpp:194-271, launched at
+ * getp_run.cpp:688-695), the layer itself as moe_forward, and
+ * residual_add_batch_kernel (utility/utility.cpp:158-173, launched at
+ * getp_run.cpp:846-852); on the CPU path run.cpp:660-750.  The normalised rows
+ * and the fp32 sum never leave the library's workspace.  Rows with pos < 0 are
+ * left as they are.  Asynchronous on `stream`. */
+int moe_block_forward(moe_handle *h, int layer, uint16_t *x, const int *pos,
+                      int n_tokens, void *stream);
+
 /* Stage 1 alone.  Writes topk_i int [n_tokens,K] (descending score, ties to
  * the lower expert id; -1 on inactive rows), topk_v f32 [n_tokens,K] (softmax
  * over the K selected logits) and, if score != NULL, the logits f32

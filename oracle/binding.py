@@ -53,6 +53,7 @@ def lib():
         L.oracle_moe_layer.argtypes = ([_f, C.c_void_p] + [_f] * 6 + [C.c_int] * 5 +
                                        [C.c_float, C.c_int, _f, C.c_void_p, C.c_void_p, C.c_void_p])
         L.oracle_mxfp4_dequant.argtypes = [_u8, _u8, C.c_size_t, _f]
+        L.oracle_rmsnorm.argtypes = [_f, _f, _f, C.c_int]
         L.oracle_num_threads.restype = C.c_int
         _lib = L
     return _lib
@@ -132,6 +133,32 @@ def moe_layer(x, pos, wr, br, w1, b1, w2, b2, K, limit, mode=0, want_routing=Fal
     return (out, score, ti, tv) if want_routing else out
 
 
+def rmsnorm(x, weight):
+    """Row-wise oracle_rmsnorm of x [T, H] (or [H])."""
+    x2 = np.ascontiguousarray(np.atleast_2d(x), np.float32)
+    w = np.ascontiguousarray(weight, np.float32)
+    out = np.empty_like(x2)
+    for t in range(x2.shape[0]):
+        lib().oracle_rmsnorm(out[t], x2[t], w, x2.shape[1])
+    return out.reshape(np.shape(x))
+
+
+def ffn_block(x, pos, rms_w, wr, br, w1, b1, w2, b2, K, limit, mode=0):
+    """The FFN block on a bf16 residual stream: t = bf16(rmsnorm(x) * w)
+    (run.cpp:660; the layer's input is bf16 on the GPU path, defines.h:107),
+    out = moe_layer(t) (run.cpp:662-745), x' = bf16(x + out) (run.cpp:748-750;
+    utility.cpp:158-173 rounds the sum to bf16).  Rows with pos < 0 keep x.
+    Returns (x', t)."""
+    x = np.ascontiguousarray(x, np.float32)
+    t = round_to_bf16(rmsnorm(x, rms_w))
+    out = moe_layer(t, pos, wr, br, w1, b1, w2, b2, K, limit, mode=mode)
+    xn = round_to_bf16(x + out)
+    if pos is not None:
+        inactive = np.asarray(pos) < 0
+        xn[inactive] = x[inactive]
+    return xn, t
+
+
 def mxfp4_dequant(blocks, scales):
     blocks = np.ascontiguousarray(blocks, np.uint8)
     scales = np.ascontiguousarray(scales, np.uint8)
@@ -162,6 +189,7 @@ def ref():
         L.ref_matmul.argtypes = [_f, _f, _f, C.c_int, C.c_int]
         L.ref_topk.argtypes = [_f, _i, _f, C.c_int, C.c_int]
         L.ref_softmax.argtypes = [_f, C.c_int]
+        L.ref_rmsnorm.argtypes = [_f, _f, _f, C.c_int]
         L.ref_moe_forward.argtypes = ([C.c_int] * 5 + [C.c_float] + [_f] * 7 + [_f, _f, _i, _f, _f])
         L.ref_moe_forward.restype = C.c_int
         _ref = L

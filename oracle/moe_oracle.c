@@ -81,6 +81,16 @@ void oracle_topk(float *topk_v, int *topk_i, const float *score, int E, int K) {
   }
 }
 
+/* ---- run.cpp:321-334 ---- */
+void oracle_rmsnorm(float *o, const float *x, const float *weight, int size) {
+  double ss = 0.0f;
+  for (int j = 0; j < size; j++) ss += x[j] * x[j]; /* float product, double sum */
+  ss /= size;
+  ss += 1e-5f;
+  ss = 1.0f / sqrtf(ss); /* the argument is narrowed to float */
+  for (int j = 0; j < size; j++) o[j] = weight[j] * (ss * x[j]);
+}
+
 /* ---- run.cpp:336-354 ---- */
 void oracle_softmax(float *x, int size) {
   double max_val = x[0];

@@ -23,6 +23,12 @@
  *         exhaustive comparison against an integer formulation.
  *   oracle_mxfp4_dequant
  *       - pinned by the 16-code x 11-exponent closed-form table.
+ *   oracle_rmsnorm
+ *       - the committed config-1 vectors hold the reference's own t =
+ *         rmsnorm(embedding row) (unit weight); compared bit for bit; with
+ *         other weights compared against the reference's rmsnorm() from
+ *         oracle/_ref where that is built; closed forms (constant vector,
+ *         invariance of the direction under scaling).
  *   oracle_moe_layer with ORACLE_ROUND_ACT_BF16
  *       - same control flow as mode 0; the extra rounding point is the one
  *         the reference's GPU path has (matmul.cpp:1427).  When the rounding
@@ -54,6 +60,8 @@ void oracle_matmul(float *xout, const float *x, const float *w, int n, int d);
 void oracle_topk(float *topk_v, int *topk_i, const float *score, int E, int K);
 /* run.cpp:336-354 */
 void oracle_softmax(float *x, int size);
+/* run.cpp:321-334: o = weight * x / sqrt(mean(x^2) + 1e-5) */
+void oracle_rmsnorm(float *o, const float *x, const float *weight, int size);
 
 /* run.cpp:664-676 for every row with pos >= 0 (pos may be NULL = all active).
  * Inactive rows: topk_i = -1, topk_v = 0, score untouched. */

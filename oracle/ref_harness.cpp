@@ -14,6 +14,9 @@
 
 extern "C" {
 
+// run.cpp:321-334
+void ref_rmsnorm(float *o, float *x, float *weight, int size) { rmsnorm(o, x, weight, size); }
+
 // run.cpp:356-369
 void ref_matmul(float *xout, float *x, float *w, int n, int d) { matmul(xout, x, w, n, d); }
 // run.cpp:388-421

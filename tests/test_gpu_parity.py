@@ -289,6 +289,49 @@ def test_c5_mxfp4_ingest():
         m4.upload_layer_mxfp4(3, wr, br, b1k, s1, b1, b2k, s2, b2)  # layer out of range
 
 
+def test_ffn_block_in_place(c2):
+    """moe_block_forward: RMS norm in front, residual add behind, in place on a
+    bf16 stream.  The norm is checked through the routing it leads to (bit-exact
+    offsets and permutation need bit-exact normalised rows up to near-ties), the
+    result against the oracle's composition of the same steps."""
+    sh, L, m = c2
+    T = 1024
+    rng = np.random.default_rng(21)
+    x = synth.round_bf16((rng.standard_normal((T, sh.hidden)) * rng.uniform(0.5, 4.0, (T, 1))).astype(np.float32))
+    rw = synth.round_bf16((1 + 0.1 * rng.standard_normal(sh.hidden)).astype(np.float32))
+    pos = np.zeros(T, np.int32)
+    pos[5::9] = -1
+    m.upload_norm(0, rw)
+    dx = abi.DevBuf.from_numpy(synth.to_bf16_bits(x))
+    dpos = abi.DevBuf.from_numpy(pos)
+    m.block_forward(0, dx, dpos, T)
+    doff, dperm = abi.DevBuf((sh.experts + 1) * 4), abi.DevBuf(T * 4 * 4)
+    m.get_dispatch(doff, dperm, T)
+    abi.sync()
+    got = synth.from_bf16_bits(dx.download((T, sh.hidden), np.uint16))
+    off = doff.download((sh.experts + 1,), np.int32)
+    perm = dperm.download((T * 4,), np.int32)
+
+    t = ob.round_to_bf16(ob.rmsnorm(x, rw))
+    _, ti, _ = ob.router(t, pos, L["w_router"], L["b_router"], 4)
+    off_o, perm_o, _ = ob.dispatch(ti, pos, sh.experts)
+    assert np.array_equal(off, off_o) and np.array_equal(perm[:off_o[-1]], perm_o)
+
+    rows = np.sort(rng.choice(T, 24, replace=False))
+    want, _ = ob.ffn_block(x[rows], pos[rows], rw, *[L[k] for k in W], 4, sh.limit,
+                           mode=ob.ROUND_ACT_BF16 | ob.PAR_TOKENS)
+    # one bf16 step of the result on top of the layer's bar
+    tol = MAX_ABS + 2.0 ** -7 * np.abs(want)
+    assert np.all(np.abs(got[rows] - want) <= tol)
+    assert rel_l2(got[rows], want) <= 4e-3  # bf16 output: 2^-9 relative rounding
+    inactive = pos < 0
+    assert np.array_equal(got[inactive], x[inactive])
+
+    m2 = abi.Moe(sh.hidden, sh.inter, sh.experts, max_tokens=64)
+    with pytest.raises(abi.MoeError):  # no weights, no norm weight
+        m2.block_forward(0, dx, None, 16)
+
+
 # ---------------- host logic on the GPU box ----------------
 
 def test_error_paths_and_profiling(c2):

@@ -72,6 +72,67 @@ def test_against_reference_build_random_shapes():
         assert np.array_equal(y, ob.matmul(x, wr))
 
 
+def test_rmsnorm_matches_reference_vectors(golden, c1_layer):
+    """The fixture's t is the reference's own rmsnorm (unit weight) of the
+    embedding rows, taken out of forward()'s state (run.cpp:660)."""
+    x = c1_layer["x"]
+    assert synth.digest(x) == str(golden["emb_digest"])
+    t = ob.rmsnorm(x, np.ones(x.shape[1], np.float32))
+    assert np.array_equal(t, golden["t"])
+
+
+@pytest.mark.skipif(not ob.ref_available(), reason="reference build (oracle/_ref) not present")
+def test_rmsnorm_against_reference_build():
+    rng = np.random.default_rng(11)
+    for H in (64, 2880, 257):
+        x = (rng.standard_normal(H) * rng.uniform(0.01, 30)).astype(np.float32)
+        w = (1 + 0.2 * rng.standard_normal(H)).astype(np.float32)
+        want = np.empty(H, np.float32)
+        ob.ref().ref_rmsnorm(want, x.copy(), w.copy(), H)
+        assert np.array_equal(ob.rmsnorm(x, w), want)
+
+
+def test_rmsnorm_closed_forms():
+    H = 96
+    w = np.linspace(0.5, 1.5, H).astype(np.float32)
+    # constant rows: mean square is c^2 exactly
+    for c in (1.0, -3.0, 0.25):
+        x = np.full(H, c, np.float32)
+        scale = np.float32(1.0) / np.sqrt(np.float32(np.float64(c) * c + np.float64(np.float32(1e-5))))
+        want = (w.astype(np.float64) * (np.float64(scale) * np.float64(c))).astype(np.float32)
+        assert np.array_equal(ob.rmsnorm(x, w), want)
+    # the direction survives scaling; the length is sqrt(H) up to the epsilon
+    rng = np.random.default_rng(3)
+    x = rng.standard_normal(H).astype(np.float32)
+    a = ob.rmsnorm(x, np.ones(H, np.float32))
+    b = ob.rmsnorm(64 * x, np.ones(H, np.float32))
+    np.testing.assert_allclose(a, b, rtol=2e-5)
+    np.testing.assert_allclose(np.linalg.norm(a.astype(np.float64)), np.sqrt(H), rtol=1e-4)
+    # a zero row stays zero (the epsilon keeps the scale finite)
+    assert np.all(ob.rmsnorm(np.zeros(H, np.float32), w) == 0)
+
+
+def test_ffn_block_composition():
+    """x' = bf16(x + layer(bf16(rmsnorm(x) w))); inactive rows keep x."""
+    rng = np.random.default_rng(8)
+    T, H, IM, E = 6, 64, 64, 8
+    x = ob.round_to_bf16((rng.standard_normal((T, H)) * 2).astype(np.float32))
+    rw = ob.round_to_bf16((1 + 0.1 * rng.standard_normal(H)).astype(np.float32))
+    wr = (rng.standard_normal((E, H)) * 0.3).astype(np.float32)
+    br = (rng.standard_normal(E) * 0.1).astype(np.float32)
+    w1 = (rng.standard_normal((E, 2 * IM, H)) * 0.1).astype(np.float32)
+    b1 = np.zeros((E, 2 * IM), np.float32)
+    w2 = np.zeros((E, H, IM), np.float32)       # experts output their bias only
+    b2 = np.full((E, H), 0.5, np.float32)
+    pos = np.array([0, 0, -1, 0, 0, 0], np.int32)
+    xn, t = ob.ffn_block(x, pos, rw, wr, br, w1, b1, w2, b2, 4, 7.0)
+    assert np.array_equal(t, ob.round_to_bf16(ob.rmsnorm(x, rw)))
+    act = pos >= 0
+    # routing weights sum to one, so the layer adds 0.5 to every element
+    np.testing.assert_allclose(xn[act], ob.round_to_bf16(x[act] + np.float32(0.5)), rtol=0, atol=2.0 ** -6)
+    assert np.array_equal(xn[~act], x[~act])
+
+
 # ---------------- what the mathematics fixes ----------------
 
 def test_matmul_one_hot_and_double_accumulation():
