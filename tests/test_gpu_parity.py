@@ -243,6 +243,34 @@ def test_c3_zipf_routing(name, c2):
         m.upload_layer(0, *[L2[k] for k in W])
 
 
+def test_all_tokens_on_four_experts_and_tiny_batches(c2):
+    """The tile plan's extremes: 28 experts without a row and four with every
+    row (the XCD ranges then cut through single experts), and batches far below
+    one tile."""
+    sh, L2, m = c2
+    L = dict(L2)
+    br = np.full(sh.experts, -30.0, np.float32)
+    br[[3, 7, 20, 31]] = [30.0, 29.0, 28.0, 27.0]
+    L["b_router"] = synth.round_bf16(br)
+    m.upload_layer(0, *[L[k] for k in W])
+    try:
+        T = 3000
+        x = L2["x"][:T]
+        R = abi.run_layer(m, 0, x, None)
+        _, off = check_routing(R, L, x, None, sh.experts)
+        counts = np.diff(off)
+        assert sorted(np.nonzero(counts)[0]) == [3, 7, 20, 31] and np.all(counts[[3, 7, 20, 31]] == T)
+        rows = np.sort(np.random.default_rng(6).choice(T, 24, replace=False))
+        check_outputs(R, L, x, None, rows)
+    finally:
+        m.upload_layer(0, *[L2[k] for k in W])
+    for T in (1, 2, 33):
+        x = L2["x"][100:100 + T]
+        R = abi.run_layer(m, 0, x, None)
+        check_routing(R, L2, x, None, sh.experts)
+        check_outputs(R, L2, x, None, np.arange(T))
+
+
 def test_c4_120b_shape():
     sh = synth.CONFIGS["c4"]
     L = bf16_layer(sh)
