@@ -86,10 +86,16 @@ __global__ __launch_bounds__(256) void dispatch_scan_kernel(int *__restrict__ bl
   const int e = threadIdx.x;
   int count = 0;
   if (e < E) {
-    for (int b = 0; b < n_blk; b++) {
-      const int c = blk_counts[(size_t)b * E + e];
-      blk_counts[(size_t)b * E + e] = count;
-      count += c;
+    // 16 independent loads at a time, then their running sums back in place
+    for (int b0 = 0; b0 < n_blk; b0 += 16) {
+      int c[16];
+#pragma unroll
+      for (int i = 0; i < 16; i++) c[i] = b0 + i < n_blk ? blk_counts[(size_t)(b0 + i) * E + e] : 0;
+#pragma unroll
+      for (int i = 0; i < 16; i++) {
+        if (b0 + i < n_blk) blk_counts[(size_t)(b0 + i) * E + e] = count;
+        count += c[i];
+      }
     }
   }
   const int n_rb = (count + kRowBlock - 1) / kRowBlock;
