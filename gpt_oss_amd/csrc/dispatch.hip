@@ -78,8 +78,12 @@ __global__ __launch_bounds__(256) void dispatch_scan_kernel(int *__restrict__ bl
                                                            int E, int n_ct_gate_up, int n_ct_down,
                                                            int *__restrict__ offsets,
                                                            ExpertInfo *__restrict__ info,
-                                                           int *__restrict__ totals) {
+                                                           int *__restrict__ totals,
+                                                           TileDesc *__restrict__ tiles_gate_up,
+                                                           TileDesc *__restrict__ tiles_down,
+                                                           int tile_cap_gate_up, int tile_cap_down) {
   __shared__ int buf[256];
+  __shared__ int sh_nmt[256], sh_rb[256], sh_extra[256], sh_rowblk[256];
   __shared__ int sh_cost[257];   // exclusive prefix of the experts' cost per column tile
   __shared__ int sh_tiles[257];  // exclusive prefix of their row tiles
   __shared__ int sh_bound[2][kXcds + 1];
@@ -126,6 +130,10 @@ __global__ __launch_bounds__(256) void dispatch_scan_kernel(int *__restrict__ bl
   const int ex_cost = block_exclusive_scan_256(cost, buf, e, &tot_cost);
   sh_cost[e] = ex_cost;
   sh_tiles[e] = ex_mt;
+  sh_nmt[e] = n_mt;
+  sh_rb[e] = rb;
+  sh_extra[e] = extra;
+  sh_rowblk[e] = ex_pad / kRowBlock;
   if (e == 0) {
     sh_cost[256] = tot_cost;
     sh_tiles[256] = tot_mt;
@@ -184,6 +192,29 @@ __global__ __launch_bounds__(256) void dispatch_scan_kernel(int *__restrict__ bl
       prev = bnd;
     }
     out[kXcds] = total_tiles;
+  }
+  // The tile sequences: tile L = (expert, column tile, row tile), row tile fastest.
+  for (int g = 0; g < 2; g++) {
+    const int n_ct = g ? n_ct_down : n_ct_gate_up;
+    TileDesc *tiles = g ? tiles_down : tiles_gate_up;
+    const int total_tiles = min(tot_mt * n_ct, g ? tile_cap_down : tile_cap_gate_up);
+    for (int L = e; L < total_tiles; L += 256) {
+      // last expert whose first tile is at or before L; experts without rows share
+      // their successor's start and are passed over
+      int lo = 0, hi = 255;
+      while (lo < hi) {
+        const int mid = (lo + hi + 1) >> 1;
+        if (sh_tiles[mid] * n_ct <= L) lo = mid; else hi = mid - 1;
+      }
+      const int rem = L - sh_tiles[lo] * n_ct;
+      const int mt = rem % sh_nmt[lo];
+      TileDesc d;
+      d.e = lo;
+      d.nt = rem / sh_nmt[lo];
+      d.rbt = sh_rb[lo] + (mt < sh_extra[lo] ? 1 : 0);
+      d.rb0 = sh_rowblk[lo] + mt * sh_rb[lo] + min(mt, sh_extra[lo]);
+      tiles[L] = d;
+    }
   }
 }
 
@@ -333,7 +364,8 @@ hipError_t launch_dispatch(const int *topk_i, const int *pos, int T, int E, int 
   dispatch_count_kernel<<<n_blk, kDispThreads, 0, s>>>(topk_i, pos, T, E, d.blk_counts, d.rowmap,
                                                        fill_rows, d.perm);
   dispatch_scan_kernel<<<1, 256, 0, s>>>(d.blk_counts, n_blk, E, n_ct_gate_up, n_ct_down, d.offsets,
-                                         d.info, d.totals);
+                                         d.info, d.totals, d.tiles_gate_up, d.tiles_down,
+                                         d.tile_cap_gate_up, d.tile_cap_down);
   dispatch_scatter_kernel<<<n_blk, kDispThreads, 0, s>>>(topk_i, pos, T, E, d.blk_counts, d.offsets,
                                                          d.info, d.perm, d.rowmap, d.inv);
   return hipGetLastError();

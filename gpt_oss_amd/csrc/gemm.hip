@@ -73,42 +73,16 @@ __device__ __forceinline__ uint32_t pack_bf16(float a, float b) {
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
-struct TileCoord {
-  int e;      // expert
-  int rb0;    // first row block (32 rows) of the tile in the padded row space
-  int nt;     // column tile
-  int rows0;  // first row of the tile relative to the expert's segment
-};
-
-// Maps the workgroup id to a tile (see "Tile order" above).  Returns false for
-// the surplus workgroups of the upper-bound grid.
-__device__ __forceinline__ bool locate_tile(const ExpertInfo *__restrict__ info,
-                                            const int *__restrict__ bounds, int E, int n_ct,
-                                            TileCoord &tc, int &rb) {
+// Maps the workgroup id to a tile (see "Tile order" above): two dependent
+// loads, the XCD's range and the tile's descriptor.  Returns false for the
+// surplus workgroups of the upper-bound grid.
+__device__ __forceinline__ bool locate_tile(const TileDesc *__restrict__ tiles,
+                                            const int *__restrict__ bounds, TileDesc &d) {
   const int bid = blockIdx.x;
   const int xcd = bid & (kXcds - 1);
-  const int first = bounds[xcd];
-  const int L = first + (bid >> 3);
+  const int L = bounds[xcd] + (bid >> 3);
   if (L >= bounds[xcd + 1]) return false;
-  // largest e with tile_base[e] * n_ct <= L and n_mt[e] > 0
-  int lo = 0, hi = E - 1;
-  while (lo < hi) {
-    const int mid = (lo + hi + 1) >> 1;
-    if (info[mid].tile_base * n_ct <= L) lo = mid; else hi = mid - 1;
-  }
-  // An expert without rows shares tile_base with its successor, so the search
-  // passes over it; a trailing run of empty experts has tile_base equal to the
-  // number of row tiles and cannot be reached because L is a valid tile.
-  const int e = lo;
-  const ExpertInfo inf = info[e];
-  const int rem = L - inf.tile_base * n_ct;
-  const int mt = rem % inf.n_mt;
-  tc.e = e;
-  tc.nt = rem / inf.n_mt;
-  rb = inf.rb + (mt < inf.extra ? 1 : 0);
-  const int rb_first = mt * inf.rb + min(mt, inf.extra);  // relative to the expert's segment
-  tc.rows0 = rb_first * kRowBlock;
-  tc.rb0 = inf.row0 / kRowBlock + rb_first;
+  d = tiles[L];
   return true;
 }
 
@@ -451,8 +425,8 @@ template <typename C, bool GATE_UP>
 __global__ __launch_bounds__(C::THREADS) void grouped_gemm_kernel(
     const uint4 *__restrict__ a_frag, const uint4 *__restrict__ w_frag,
     const float *__restrict__ bias_a, const float *__restrict__ bias_b,
-    const ExpertInfo *__restrict__ info, const int *__restrict__ totals, void *__restrict__ outp,
-    int K, int N, int E, float limit) {
+    const TileDesc *__restrict__ tiles, const int *__restrict__ totals, void *__restrict__ outp,
+    int K, int N, float limit) {
   constexpr int R = C::R;
   static_assert(R == 7, "seven stage arrays are declared below");
   __shared__ uint4 st0[C::STAGE], st1[C::STAGE], st2[C::STAGE], st3[C::STAGE], st4[C::STAGE],
@@ -461,9 +435,8 @@ __global__ __launch_bounds__(C::THREADS) void grouped_gemm_kernel(
   const int KB = K / kFragK;
   const int nb_total = (GATE_UP ? 2 * N : N) / kRowBlock;  // weight row blocks per expert
   const int n_ct = (nb_total + C::TILE_NB - 1) / C::TILE_NB;
-  TileCoord tc;
-  int rb;
-  if (!locate_tile(info, totals + (GATE_UP ? kTotBoundsGateUp : kTotBoundsDown), E, n_ct, tc, rb)) return;
+  TileDesc tc;
+  if (!locate_tile(tiles, totals + (GATE_UP ? kTotBoundsGateUp : kTotBoundsDown), tc)) return;
   const int nb0 = tc.nt * C::TILE_NB;
   const int nb_valid = min(C::TILE_NB, nb_total - nb0);
   const uint4 *b_frag = w_frag + (size_t)tc.e * nb_total * KB * 64;
@@ -471,7 +444,7 @@ __global__ __launch_bounds__(C::THREADS) void grouped_gemm_kernel(
   const float *bb = GATE_UP ? bias_b + (size_t)tc.e * N : nullptr;
 #define MOE_TILE_CASE(n) \
   case n: gemm_tile<n, C, GATE_UP>(a_frag, b_frag, KB, tc.rb0, nb0, nb_valid, ba, bb, outp, N, limit, st0, st1, st2, st3, st4, st5, st6, epi); break;
-  switch (rb) {
+  switch (tc.rbt) {
     MOE_TILE_CASE(1) MOE_TILE_CASE(2) MOE_TILE_CASE(3) MOE_TILE_CASE(4)
     MOE_TILE_CASE(5) MOE_TILE_CASE(6) MOE_TILE_CASE(7)
     default: gemm_tile<8, C, GATE_UP>(a_frag, b_frag, KB, tc.rb0, nb0, nb_valid, ba, bb, outp, N, limit, st0, st1, st2, st3, st4, st5, st6, epi); break;
@@ -492,8 +465,9 @@ static hipError_t launch_gemm(const uint4 *a, const uint4 *w, const float *ba, c
   const int nb_total = (GATE_UP ? 2 * N : N) / kRowBlock;
   const int n_ct = (nb_total + C::TILE_NB - 1) / C::TILE_NB;
   const int grid = kXcds * xcd_tile_cap(mt_cap * n_ct);
-  grouped_gemm_kernel<C, GATE_UP><<<grid, C::THREADS, 0, s>>>(a, w, ba, bb, d.info, d.totals, out, K,
-                                                              N, E, limit);
+  (void)E;
+  grouped_gemm_kernel<C, GATE_UP><<<grid, C::THREADS, 0, s>>>(
+      a, w, ba, bb, GATE_UP ? d.tiles_gate_up : d.tiles_down, d.totals, out, K, N, limit);
   return hipGetLastError();
 }
 

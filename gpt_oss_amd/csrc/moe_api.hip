@@ -204,6 +204,13 @@ int moe_create(const moe_config *cfg, moe_handle **out) {
   ALLOC(h->disp.inv, (size_t)h->a_cap);
   ALLOC(h->disp.info, (size_t)E);
   ALLOC(h->disp.totals, (size_t)kTotInts);
+  {
+    const int mt_cap = h->a_cap / kTileRows + E;  // row tiles at max_tokens, at most
+    h->disp.tile_cap_gate_up = mt_cap * gate_up_col_tiles(*cfg);
+    h->disp.tile_cap_down = mt_cap * down_col_tiles(*cfg);
+  }
+  ALLOC(h->disp.tiles_gate_up, (size_t)h->disp.tile_cap_gate_up);
+  ALLOC(h->disp.tiles_down, (size_t)h->disp.tile_cap_down);
   ALLOC(h->xg, (size_t)h->a_pad_cap * H);
   ALLOC(h->act, (size_t)h->a_pad_cap * IM);
   ALLOC(h->y, (size_t)h->a_pad_cap * H);
@@ -229,6 +236,7 @@ int moe_destroy(moe_handle *h) {
   (void)hipFree(h->topk_i); (void)hipFree(h->topk_v);
   (void)hipFree(h->disp.blk_counts); (void)hipFree(h->disp.offsets); (void)hipFree(h->disp.perm);
   (void)hipFree(h->disp.rowmap); (void)hipFree(h->disp.inv); (void)hipFree(h->disp.info); (void)hipFree(h->disp.totals);
+  (void)hipFree(h->disp.tiles_gate_up); (void)hipFree(h->disp.tiles_down);
   (void)hipFree(h->xg); (void)hipFree(h->act); (void)hipFree(h->y); (void)hipFree(h->t_norm);
   for (hipEvent_t ev : h->events) (void)hipEventDestroy(ev);
   delete h;

@@ -52,6 +52,17 @@ struct ExpertInfo {
   int pad_[2];
 };
 
+// One tile of a grouped GEMM, looked up by its number in the tile sequence.
+// Written by the scan kernel for both GEMMs, so that a GEMM workgroup finds its
+// work with one load instead of a binary search over the experts (a chain of
+// dependent global loads in front of every tile).
+struct TileDesc {
+  int e;    // expert
+  int rb0;  // first row block of the tile in the padded row space
+  int rbt;  // its row blocks (1..8)
+  int nt;   // column tile
+};
+
 struct LayerWeights {
   uint16_t *wr = nullptr;  // router weight, bf16 in the operand order of the f64 MFMA
   float *br = nullptr;     // router bias, padded experts = -inf
@@ -88,6 +99,9 @@ struct DispatchBuffers {
   ExpertInfo *info;   // [E]
   int *totals;        // [kTotInts]: total row tiles, padded rows, assignments; XCD bounds of both GEMMs
   int a_pad_cap;      // capacity of rowmap in rows
+  TileDesc *tiles_gate_up;  // [tile_cap_gate_up] tile sequence of the gate_up GEMM
+  TileDesc *tiles_down;     // [tile_cap_down]    ... of the down GEMM
+  int tile_cap_gate_up, tile_cap_down;
 };
 hipError_t launch_dispatch(const int *topk_i, const int *pos, int T, int E, int n_ct_gate_up,
                            int n_ct_down, const DispatchBuffers &d, hipStream_t s);
