@@ -360,6 +360,48 @@ def test_ffn_block_in_place(c2):
         m2.block_forward(0, dx, None, 16)
 
 
+def test_forward_replays_from_a_hip_graph(c2):
+    """moe_forward allocates nothing, never synchronises and clears its buffers
+    with kernels, so a caller may capture it.  Three replays, with eager calls
+    and synchronisations of the program's own in between, must each reproduce the
+    eager result bit for bit."""
+    import ctypes as C
+    hip = C.CDLL("libamdhip64.so")
+
+    def ok(rc):
+        assert rc == 0, f"HIP call failed with {rc}"
+
+    sh, L, m = c2
+    T = 1500
+    x = L["x"][:T]
+    dx = abi.DevBuf.from_numpy(synth.to_bf16_bits(x))
+    dout, dref = abi.DevBuf(T * sh.hidden * 4), abi.DevBuf(T * sh.hidden * 4)
+    stream = C.c_void_p()
+    ok(hip.hipStreamCreate(C.byref(stream)))
+    m.forward(0, dx, None, T, dref, stream=stream)
+    ok(hip.hipStreamSynchronize(stream))
+    ref = dref.download((T, sh.hidden), np.float32)
+    graph, gexec = C.c_void_p(), C.c_void_p()
+    ok(hip.hipStreamBeginCapture(stream, C.c_int(0)))
+    m.forward(0, dx, None, T, dout, stream=stream)
+    ok(hip.hipStreamEndCapture(stream, C.byref(graph)))
+    ok(hip.hipGraphInstantiate(C.byref(gexec), graph, None, None, C.c_size_t(0)))
+    try:
+        for _ in range(3):
+            dout.memset(0)
+            abi.sync()
+            ok(hip.hipGraphLaunch(gexec, stream))
+            ok(hip.hipStreamSynchronize(stream))
+            assert np.array_equal(dout.download((T, sh.hidden), np.float32), ref)
+            # eager work of a different size between the replays
+            m.forward(0, dx, None, T // 2, dref, stream=stream)
+            ok(hip.hipStreamSynchronize(stream))
+    finally:
+        hip.hipGraphExecDestroy(gexec)
+        hip.hipGraphDestroy(graph)
+        hip.hipStreamDestroy(stream)
+
+
 # ---------------- host logic on the GPU box ----------------
 
 def test_error_paths_and_profiling(c2):
