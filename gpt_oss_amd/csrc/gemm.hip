@@ -15,9 +15,9 @@
 // 1..8 following the expert's row count (see dispatch_scan_kernel), so a ragged
 // segment pads to at most 31 rows and MFMA work follows the real rows.
 //
-// Feeding the matrix cores.  What bounds this kernel is how fast one CU can
-// take data in from L2 (about 45 GB/s with 100 KB in flight, 55-60 GB/s with
-// 200 KB), so the design maximises bytes in flight:
+// Feeding the matrix cores.  A step of 32 k needs 32 KB per CU, and one CU
+// takes data in from L2 at about 45 GB/s with 100 KB in flight and 55-60 GB/s
+// with 200 KB, so the design keeps many bytes in flight:
 //   * the row operand (shared by all waves) goes straight into an R-stage LDS
 //     ring by DMA (global_load_lds_dwordx4), R-1 steps ahead of the MFMAs;
 //   * the column operand is private to a wave in this layout, so it never
@@ -25,6 +25,8 @@
 // With R = 7 that is 6 steps x 32 KB = 192 KB in flight per CU.  Loads return
 // in order, so waiting for "all but the newest n" (s_waitcnt vmcnt(n)) picks out
 // exactly the step that is needed next and leaves the later ones in flight.
+// Measured in the steady loop: 1113 clocks per step of 1024 MFMA clocks (tile of
+// 8 row blocks), the same in every group of every tile.
 //
 // Tile order.  Workgroup ids are dealt round-robin to the 8 XCDs, each with
 // its own L2.  Logical tile ids are laid out (expert, column tile, row tile)
@@ -43,12 +45,6 @@ using IC = std::integral_constant<int, V>;
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
-
-__device__ __forceinline__ uint16_t f32_to_bf16_rne_dev(float f) {
-  uint32_t u = __float_as_uint(f);
-  u += 0x7fffu + ((u >> 16) & 1u);  // finite inputs only
-  return (uint16_t)(u >> 16);
-}
 
 // run.cpp:709-726: gate clamped from above, up clamped on both sides, then
 // gate * sigmoid(alpha * gate) * (up + 1).  u1 is up + 1 already (the 1 rides
