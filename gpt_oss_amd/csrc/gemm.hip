@@ -124,9 +124,18 @@ struct GemmCfg {
   static constexpr int EPI_WAVE = 32 * EPI_LD / 4;       // uint4 per wave of epilogue buffer
 };
 
-template <int RBT, typename C, bool GATE_UP>
+// FP4: the column operand is MXFP4 as packed by pack_fp4_kernel: per pair of
+// column blocks and step of 32 k one 16-byte chunk per lane (blocks 2P and 2P+1,
+// each [k block 0: 8 nibbles][k block 1: 8 nibbles] of the lane's row) and two
+// scale bytes per row.  A step of 32 k is exactly one MXFP4 block, so one scale
+// serves both of its k blocks.  The nibbles become bf16 MFMA operands in
+// registers (v_cvt_scalef32_pk_bf16_fp4: two values and their scale per
+// instruction, exact); everything else is the bf16 kernel, which then takes in
+// 4.25 KB instead of 16 KB of weights per CU and step.
+template <int RBT, typename C, bool GATE_UP, bool FP4>
 __device__ __forceinline__ void gemm_tile(const uint4 *__restrict__ a_frag,  // [rb][KB][64]
-                                          const uint4 *__restrict__ b_frag,  // expert: [nb][KB][64]
+                                          const uint4 *__restrict__ b_frag,  // expert: [nb][KB][64], FP4: [nb/2][KB/2][64]
+                                          const uint16_t *__restrict__ b_scale,  // FP4: expert's [nb/2][KB/2][32] byte pairs
                                           int KB, int rb0, int nb0, int nb_valid,
                                           const float *__restrict__ bias_a,  // gate / down bias (expert)
                                           const float *__restrict__ bias_b,  // up bias (expert)
@@ -151,11 +160,14 @@ __device__ __forceinline__ void gemm_tile(const uint4 *__restrict__ a_frag,  // 
   static_assert(KPS == 2, "the step is software-pipelined as two k blocks");
   constexpr int A_CH = RBT * KPS;            // 1 KB chunks of the row operand per step
   constexpr int LA = (A_CH + NW - 1) / NW;   // DMA loads per wave per step (a short last pass repeats a chunk)
-  constexpr int LB = NBW * KPS;              // register loads per wave per step
+  constexpr int LB = FP4 ? 2 : NBW * KPS;    // register loads per wave per step
   constexpr int LPS = LA + LB;
   static_assert(LPS * (R - 2) + LA <= 63, "vmcnt is a 6-bit counter");
+  static_assert(!FP4 || NBW == 2, "an MXFP4 chunk holds the pair of column blocks of one wave");
   constexpr int NM = RBT * NBW;              // MFMAs per k block
-  constexpr int SIDE = (RBT + LB + NM - 1) / NM;  // side items per MFMA
+  constexpr int DEC = FP4 ? NBW : 0;         // decode items per k block (one column block each)
+  constexpr int SIDE1 = (RBT + LB + DEC + NM - 1) / NM;  // side items per MFMA, k block 0
+  constexpr int SIDE2 = (LA + RBT + DEC + NM - 1) / NM;  // ... k block 1
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -190,13 +202,21 @@ __device__ __forceinline__ void gemm_tile(const uint4 *__restrict__ a_frag,  // 
   }
   f32x16 acc[RBT][NBW];
 
+  const int n_steps = KB / KPS;
   const uint4 *a_src = a_frag + (size_t)rb0 * KB * 64 + lane;
   // Column blocks past the end of the matrix (last column tile only) re-load
   // the last valid block; their products are never stored.
   const uint4 *b_src[NBW];
+  const uint16_t *s_src = nullptr;
+  if (FP4) {
+    const size_t pair = (size_t)((nb0 + min(w * NBW, nb_valid - NBW)) >> 1);
+    b_src[0] = b_frag + pair * n_steps * 64 + lane;
+    s_src = b_scale + pair * n_steps * 32 + (lane & 31);
+  } else {
 #pragma unroll
-  for (int j = 0; j < NBW; j++)
-    b_src[j] = b_frag + (size_t)(nb0 + min(w * NBW + j, nb_valid - 1)) * KB * 64 + lane;
+    for (int j = 0; j < NBW; j++)
+      b_src[j] = b_frag + (size_t)(nb0 + min(w * NBW + j, nb_valid - 1)) * KB * 64 + lane;
+  }
 
   // Row operand: chunk c of a step (c = pass*NW + wave) is row block c / KPS, k block c % KPS.
   auto issue_a = [&](uint4 *st, int ks, int m) {
@@ -204,9 +224,32 @@ __device__ __forceinline__ void gemm_tile(const uint4 *__restrict__ a_frag,  // 
     dma_to_lds_16(a_src + ((size_t)(c / KPS) * KB + ks * KPS + c % KPS) * 64, st + c * 64);
   };
   // Column operand: register m of a slot is column block m / KPS, k block m % KPS.
-  u32x4 bq[R][LB];
+  // FP4: load 0 of a slot is the chunk of nibbles, load 1 the two scale bytes.
+  u32x4 bq[R][FP4 ? 1 : LB];
+  uint32_t bsc[R];
   auto issue_b = [&](int slot, int ks, int m) {
-    bq[slot][m] = *reinterpret_cast<const u32x4 *>(b_src[m / KPS] + (size_t)(ks * KPS + m % KPS) * 64);
+    if (FP4) {
+      if (m == 0) {
+        bq[slot][0] = *reinterpret_cast<const u32x4 *>(b_src[0] + (size_t)ks * 64);
+      } else {
+        bsc[slot] = s_src[(size_t)ks * 32];
+      }
+    } else {
+      bq[slot][m] = *reinterpret_cast<const u32x4 *>(b_src[m / KPS] + (size_t)(ks * KPS + m % KPS) * 64);
+    }
+  };
+  // FP4: the decoded operands of the step at hand, [column block][k block].
+  // Those of k block 0 are decoded during the previous step's second half,
+  // those of k block 1 during this step's first half.
+  bf16x8 bdec[NBW][KPS];
+  auto decode = [&](int slot, int j, int kk) {
+    const float scale = __uint_as_float(((bsc[slot] >> (8 * j)) & 0xffu) << 23);  // 2^(s - 127)
+    const uint32_t nib = bq[slot][0][j * KPS + kk];
+    const bf16x2 p0 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(nib, scale, 0);
+    const bf16x2 p1 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(nib, scale, 1);
+    const bf16x2 p2 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(nib, scale, 2);
+    const bf16x2 p3 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(nib, scale, 3);
+    bdec[j][kk] = bf16x8{p0[0], p0[1], p1[0], p1[1], p2[0], p2[1], p3[0], p3[1]};
   };
   // Two register sets of row fragments: while the MFMAs of one k block run, the
   // fragments of the next are read from LDS.
@@ -214,10 +257,17 @@ __device__ __forceinline__ void gemm_tile(const uint4 *__restrict__ a_frag,  // 
   auto read_a = [&](const uint4 *st, int kk, int buf, int i) {
     fa[buf][i] = __builtin_bit_cast(bf16x8, st[(i * KPS + kk) * 64 + lane]);
   };
-  auto mma = [](bf16x8 rows, u32x4 cols, f32x16 c) {
-    const bf16x8 colv = __builtin_bit_cast(bf16x8, cols);
+  auto mma = [](bf16x8 rows, bf16x8 colv, f32x16 c) {
     return GATE_UP ? __builtin_amdgcn_mfma_f32_32x32x16_bf16(colv, rows, c, 0, 0, 0)
                    : __builtin_amdgcn_mfma_f32_32x32x16_bf16(rows, colv, c, 0, 0, 0);
+  };
+  // column operand of (slot, column block j, k block kk)
+  auto cols_of = [&](int slot, int j, int kk) {
+    if constexpr (FP4) {
+      return bdec[j][kk];
+    } else {
+      return __builtin_bit_cast(bf16x8, bq[slot][j * KPS + kk]);
+    }
   };
   // "all but the newest k steps have landed", k = 0 .. R-2
 #define MOE_WAIT_STEPS(k)                            \
@@ -233,7 +283,6 @@ __device__ __forceinline__ void gemm_tile(const uint4 *__restrict__ a_frag,  // 
 
   // Issue order per wave: A(0) B(0) A(1) B(1) ... ; at the top of step ks the row
   // operand is issued through step ks+R-1 and the column operand through ks+R-2.
-  const int n_steps = KB / KPS;
 #pragma unroll
   for (int s = 0; s < R - 1; s++) {
     if (s < n_steps) {
@@ -274,6 +323,10 @@ __device__ __forceinline__ void gemm_tile(const uint4 *__restrict__ a_frag,  // 
   lds_barrier();
 #pragma unroll
   for (int i = 0; i < RBT; i++) read_a(ring.p[0], 0, 0, i);
+  if (FP4) {
+#pragma unroll
+    for (int j = 0; j < NBW; j++) decode(0, j, 0);
+  }
 
   // Step ks, slot u = ks % R:
   //   [MFMAs of k block 0 | read row fragments of k block 1, load B(ks+R-1) into slot u-1]
@@ -291,14 +344,16 @@ __device__ __forceinline__ void gemm_tile(const uint4 *__restrict__ a_frag,  // 
 #pragma unroll
     for (int m = 0; m < NM; m++) {
 #pragma unroll
-      for (int t = m * SIDE; t < (m + 1) * SIDE; t++) {
+      for (int t = m * SIDE1; t < (m + 1) * SIDE1; t++) {
         if (t < RBT) {
           read_a(cur, 1, 1, t);
         } else if (t < RBT + LB) {
           if (refill_b) issue_b((u + R - 1) % R, ks + R - 1, t - RBT);
+        } else if (t < RBT + LB + DEC) {
+          decode(u, t - RBT - LB, 1);
         }
       }
-      acc[m / NBW][m % NBW] = mma(fa[0][m / NBW], bq[u][(m % NBW) * KPS + 0], acc[m / NBW][m % NBW]);
+      acc[m / NBW][m % NBW] = mma(fa[0][m / NBW], cols_of(u, m % NBW, 0), acc[m / NBW][m % NBW]);
       __builtin_amdgcn_sched_barrier(0);
     }
     const bool more = STEADY || ks + 1 < n_steps;
@@ -316,14 +371,16 @@ __device__ __forceinline__ void gemm_tile(const uint4 *__restrict__ a_frag,  // 
 #pragma unroll
     for (int m = 0; m < NM; m++) {
 #pragma unroll
-      for (int t = m * SIDE; t < (m + 1) * SIDE; t++) {
+      for (int t = m * SIDE2; t < (m + 1) * SIDE2; t++) {
         if (t < LA) {
           if (refill_a) issue_a(ring.p[u], ks + R, t);
         } else if (t < LA + RBT) {
           if (more) read_a(nxt, 0, 0, t - LA);
+        } else if (t < LA + RBT + DEC) {
+          if (more) decode((u + 1) % R, t - LA - RBT, 0);  // landed: the wait above covers it
         }
       }
-      acc[m / NBW][m % NBW] = mma(fa[1][m / NBW], bq[u][(m % NBW) * KPS + 1], acc[m / NBW][m % NBW]);
+      acc[m / NBW][m % NBW] = mma(fa[1][m / NBW], cols_of(u, m % NBW, 1), acc[m / NBW][m % NBW]);
       __builtin_amdgcn_sched_barrier(0);
     }
   };
@@ -417,9 +474,10 @@ __device__ __forceinline__ void gemm_tile(const uint4 *__restrict__ a_frag,  // 
   }
 }
 
-template <typename C, bool GATE_UP>
+template <typename C, bool GATE_UP, bool FP4>
 __global__ __launch_bounds__(C::THREADS) void grouped_gemm_kernel(
     const uint4 *__restrict__ a_frag, const uint4 *__restrict__ w_frag,
+    const uint16_t *__restrict__ w_scale,
     const float *__restrict__ bias_a, const float *__restrict__ bias_b,
     const TileDesc *__restrict__ tiles, const int *__restrict__ totals, void *__restrict__ outp,
     int K, int N, float limit) {
@@ -435,15 +493,17 @@ __global__ __launch_bounds__(C::THREADS) void grouped_gemm_kernel(
   if (!locate_tile(tiles, totals + (GATE_UP ? kTotBoundsGateUp : kTotBoundsDown), tc)) return;
   const int nb0 = tc.nt * C::TILE_NB;
   const int nb_valid = min(C::TILE_NB, nb_total - nb0);
-  const uint4 *b_frag = w_frag + (size_t)tc.e * nb_total * KB * 64;
+  // per expert: bf16 nb_total * KB fragments of 1 KB; MXFP4 (nb_total/2) * (KB/2) chunks of 1 KB
+  const uint4 *b_frag = w_frag + (size_t)tc.e * nb_total * KB * (FP4 ? 16 : 64);
+  const uint16_t *b_scale = FP4 ? w_scale + (size_t)tc.e * nb_total * KB * 8 : nullptr;
   const float *ba = bias_a + (size_t)tc.e * N;
   const float *bb = GATE_UP ? bias_b + (size_t)tc.e * N : nullptr;
 #define MOE_TILE_CASE(n) \
-  case n: gemm_tile<n, C, GATE_UP>(a_frag, b_frag, KB, tc.rb0, nb0, nb_valid, ba, bb, outp, N, limit, st0, st1, st2, st3, st4, st5, st6, epi); break;
+  case n: gemm_tile<n, C, GATE_UP, FP4>(a_frag, b_frag, b_scale, KB, tc.rb0, nb0, nb_valid, ba, bb, outp, N, limit, st0, st1, st2, st3, st4, st5, st6, epi); break;
   switch (tc.rbt) {
     MOE_TILE_CASE(1) MOE_TILE_CASE(2) MOE_TILE_CASE(3) MOE_TILE_CASE(4)
     MOE_TILE_CASE(5) MOE_TILE_CASE(6) MOE_TILE_CASE(7)
-    default: gemm_tile<8, C, GATE_UP>(a_frag, b_frag, KB, tc.rb0, nb0, nb_valid, ba, bb, outp, N, limit, st0, st1, st2, st3, st4, st5, st6, epi); break;
+    default: gemm_tile<8, C, GATE_UP, FP4>(a_frag, b_frag, b_scale, KB, tc.rb0, nb0, nb_valid, ba, bb, outp, N, limit, st0, st1, st2, st3, st4, st5, st6, epi); break;
   }
 #undef MOE_TILE_CASE
 }
@@ -454,33 +514,39 @@ using CfgGemm = GemmCfg<4, 2, 7>;
 static_assert(CfgGemm::RBT_MAX * kRowBlock == kTileRows && CfgGemm::TILE_NB == kGemmTileNb,
               "tile plan of dispatch_scan_kernel");
 
+// w_scale == nullptr: w holds bf16 fragments; otherwise w holds MXFP4 chunks and
+// w_scale their scale bytes (pack_fp4_kernel).
 template <typename C, bool GATE_UP>
-static hipError_t launch_gemm(const uint4 *a, const uint4 *w, const float *ba, const float *bb,
-                              const DispatchBuffers &d, void *out, int K, int N, int E, float limit,
-                              int mt_cap, hipStream_t s) {
+static hipError_t launch_gemm(const uint4 *a, const uint4 *w, const uint16_t *w_scale, const float *ba,
+                              const float *bb, const DispatchBuffers &d, void *out, int K, int N,
+                              float limit, int mt_cap, hipStream_t s) {
   const int nb_total = (GATE_UP ? 2 * N : N) / kRowBlock;
   const int n_ct = (nb_total + C::TILE_NB - 1) / C::TILE_NB;
   const int grid = kXcds * xcd_tile_cap(mt_cap * n_ct);
-  (void)E;
-  grouped_gemm_kernel<C, GATE_UP><<<grid, C::THREADS, 0, s>>>(
-      a, w, ba, bb, GATE_UP ? d.tiles_gate_up : d.tiles_down, d.totals, out, K, N, limit);
+  const TileDesc *tiles = GATE_UP ? d.tiles_gate_up : d.tiles_down;
+  if (w_scale) {
+    grouped_gemm_kernel<C, GATE_UP, true><<<grid, C::THREADS, 0, s>>>(a, w, w_scale, ba, bb, tiles,
+                                                                     d.totals, out, K, N, limit);
+  } else {
+    grouped_gemm_kernel<C, GATE_UP, false><<<grid, C::THREADS, 0, s>>>(a, w, nullptr, ba, bb, tiles,
+                                                                      d.totals, out, K, N, limit);
+  }
   return hipGetLastError();
 }
 
-hipError_t launch_gate_up(const uint16_t *xg, const uint16_t *w1, const float *b1g, const float *b1u,
-                          const DispatchBuffers &d, uint16_t *act, int H, int IM, int E, float limit,
-                          int mt_cap, hipStream_t s) {
+hipError_t launch_gate_up(const uint16_t *xg, const void *w1, const uint16_t *w1_scale,
+                          const float *b1g, const float *b1u, const DispatchBuffers &d, uint16_t *act,
+                          int H, int IM, float limit, int mt_cap, hipStream_t s) {
   return launch_gemm<CfgGemm, true>(reinterpret_cast<const uint4 *>(xg),
-                                    reinterpret_cast<const uint4 *>(w1), b1g, b1u, d, act, H, IM, E,
-                                    limit, mt_cap, s);
+                                    reinterpret_cast<const uint4 *>(w1), w1_scale, b1g, b1u, d, act, H,
+                                    IM, limit, mt_cap, s);
 }
 
-hipError_t launch_down(const uint16_t *act, const uint16_t *w2, const float *b2,
-                       const DispatchBuffers &d, float *y, int H, int IM, int E, int mt_cap,
-                       hipStream_t s) {
+hipError_t launch_down(const uint16_t *act, const void *w2, const uint16_t *w2_scale, const float *b2,
+                       const DispatchBuffers &d, float *y, int H, int IM, int mt_cap, hipStream_t s) {
   return launch_gemm<CfgGemm, false>(reinterpret_cast<const uint4 *>(act),
-                                     reinterpret_cast<const uint4 *>(w2), b2, nullptr, d, y, IM, H, E,
-                                     0.f, mt_cap, s);
+                                     reinterpret_cast<const uint4 *>(w2), w2_scale, b2, nullptr, d, y,
+                                     IM, H, 0.f, mt_cap, s);
 }
 
 }  // namespace moe

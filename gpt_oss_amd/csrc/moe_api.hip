@@ -139,10 +139,11 @@ int run_experts(moe_handle *h, int layer, const uint16_t *x, const int *pos, con
   HIP_TRY(tm.mark(MOE_STAGE_GATHER));
   HIP_TRY(launch_gather(x, h->disp, h->xg, T, c.hidden, rb_cap, s));
   HIP_TRY(tm.mark(MOE_STAGE_GATE_UP));
-  HIP_TRY(launch_gate_up(h->xg, lw.w1, lw.b1g, lw.b1u, h->disp, h->act, c.hidden, c.inter,
-                         c.experts, c.swiglu_limit, mt_cap, s));
+  HIP_TRY(launch_gate_up(h->xg, lw.w1q ? static_cast<const void *>(lw.w1q) : lw.w1, lw.w1s, lw.b1g,
+                         lw.b1u, h->disp, h->act, c.hidden, c.inter, c.swiglu_limit, mt_cap, s));
   HIP_TRY(tm.mark(MOE_STAGE_DOWN));
-  HIP_TRY(launch_down(h->act, lw.w2, lw.b2, h->disp, h->y, c.hidden, c.inter, c.experts, mt_cap, s));
+  HIP_TRY(launch_down(h->act, lw.w2q ? static_cast<const void *>(lw.w2q) : lw.w2, lw.w2s, lw.b2,
+                      h->disp, h->y, c.hidden, c.inter, mt_cap, s));
   HIP_TRY(tm.mark(MOE_STAGE_COMBINE));
   if (out) {
     HIP_TRY(launch_combine(h->y, h->disp.inv, topk_v, pos, out, T, c.hidden, accumulate, s));
@@ -232,6 +233,7 @@ int moe_destroy(moe_handle *h) {
   for (auto &lw : h->layers) {
     (void)hipFree(lw.wr); (void)hipFree(lw.br); (void)hipFree(lw.w1); (void)hipFree(lw.b1g);
     (void)hipFree(lw.b1u); (void)hipFree(lw.w2); (void)hipFree(lw.b2); (void)hipFree(lw.rms_w);
+    (void)hipFree(lw.w1q); (void)hipFree(lw.w1s); (void)hipFree(lw.w2q); (void)hipFree(lw.w2s);
   }
   (void)hipFree(h->topk_i); (void)hipFree(h->topk_v);
   (void)hipFree(h->disp.blk_counts); (void)hipFree(h->disp.offsets); (void)hipFree(h->disp.perm);
@@ -260,13 +262,33 @@ int upload_layer(moe_handle *h, int layer, const float *w_router, const float *b
   int rc = MOE_OK;
 #define ALLOCW(ptr, count)                                             \
   if (rc == MOE_OK && !(ptr)) rc = dev_alloc(h, &(ptr), (count), false)
+  // MXFP4 sources stay MXFP4 on the device: a quarter of the bytes, and the
+  // GEMMs decode them in registers.
+  const bool keep_fp4 = src.mxfp4;
+  const size_t n1 = (size_t)2 * IM * H, n2 = (size_t)H * IM;  // elements of one expert's matrices
+  // a layer uploaded again in the other format gives the old copy back
+  if (keep_fp4) {
+    (void)hipFree(lw.w1); (void)hipFree(lw.w2);
+    lw.w1 = lw.w2 = nullptr;
+  } else {
+    (void)hipFree(lw.w1q); (void)hipFree(lw.w1s); (void)hipFree(lw.w2q); (void)hipFree(lw.w2s);
+    lw.w1q = lw.w2q = nullptr;
+    lw.w1s = lw.w2s = nullptr;
+  }
   ALLOCW(lw.wr, (size_t)E_pad * H);
   ALLOCW(lw.br, (size_t)E_pad);
-  ALLOCW(lw.w1, (size_t)E * 2 * IM * H);
   ALLOCW(lw.b1g, (size_t)E * IM);
   ALLOCW(lw.b1u, (size_t)E * IM);
-  ALLOCW(lw.w2, (size_t)E * H * IM);
   ALLOCW(lw.b2, (size_t)E * H);
+  if (keep_fp4) {
+    ALLOCW(lw.w1q, (size_t)E * n1 / 2);
+    ALLOCW(lw.w1s, (size_t)E * n1 / 64);  // two scale bytes per uint16
+    ALLOCW(lw.w2q, (size_t)E * n2 / 2);
+    ALLOCW(lw.w2s, (size_t)E * n2 / 64);
+  } else {
+    ALLOCW(lw.w1, (size_t)E * n1);
+    ALLOCW(lw.w2, (size_t)E * n2);
+  }
 #undef ALLOCW
   if (rc != MOE_OK) return rc;
 
@@ -295,7 +317,6 @@ int upload_layer(moe_handle *h, int layer, const float *w_router, const float *b
     // the staging buffer holds either an fp32 matrix or, in its place, the
     // (eight times smaller) blocks followed by the scales of an MXFP4 matrix
     uint8_t *stage_u8 = reinterpret_cast<uint8_t *>(stage);
-    const size_t n1 = (size_t)2 * IM * H, n2 = (size_t)H * IM;
     for (int ex = 0; ex < E; ex++) {
       if (!src.mxfp4) {
         HIP_TRY(hipMemcpy(stage, src.w1 + ex * n1, n1 * sizeof(float), hipMemcpyHostToDevice));
@@ -308,14 +329,14 @@ int upload_layer(moe_handle *h, int layer, const float *w_router, const float *b
         HIP_TRY(hipMemcpy(stage_u8, src.w1_blocks + ex * (n1 / 2), n1 / 2, hipMemcpyHostToDevice));
         HIP_TRY(hipMemcpy(stage_u8 + n1 / 2, src.w1_scales + ex * (n1 / 32), n1 / 32,
                           hipMemcpyHostToDevice));
-        HIP_TRY(launch_pack_weight_mxfp4(stage_u8, stage_u8 + n1 / 2, lw.w1 + ex * n1, 2 * IM, H, true,
-                                         nullptr));
+        HIP_TRY(launch_pack_fp4(stage_u8, stage_u8 + n1 / 2, lw.w1q + ex * (n1 / 2),
+                                lw.w1s + ex * (n1 / 64), 2 * IM, H, true, nullptr));
         HIP_TRY(hipDeviceSynchronize());
         HIP_TRY(hipMemcpy(stage_u8, src.w2_blocks + ex * (n2 / 2), n2 / 2, hipMemcpyHostToDevice));
         HIP_TRY(hipMemcpy(stage_u8 + n2 / 2, src.w2_scales + ex * (n2 / 32), n2 / 32,
                           hipMemcpyHostToDevice));
-        HIP_TRY(launch_pack_weight_mxfp4(stage_u8, stage_u8 + n2 / 2, lw.w2 + ex * n2, H, IM, false,
-                                         nullptr));
+        HIP_TRY(launch_pack_fp4(stage_u8, stage_u8 + n2 / 2, lw.w2q + ex * (n2 / 2),
+                                lw.w2s + ex * (n2 / 64), H, IM, false, nullptr));
         HIP_TRY(hipDeviceSynchronize());
       }
     }

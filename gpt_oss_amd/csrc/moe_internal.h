@@ -71,6 +71,11 @@ struct LayerWeights {
   float *b1u = nullptr;    // up bias   [E, IM]
   uint16_t *w2 = nullptr;  // down weight, bf16 MFMA fragments
   float *b2 = nullptr;     // down bias [E, H]
+  // Expert matrices kept as MXFP4 instead (moe_upload_layer_mxfp4): 16-byte
+  // chunks of nibbles and two scale bytes per row, pair of row blocks and 32 k
+  // (see pack_fp4_kernel); w1/w2 are then not allocated.
+  uint8_t *w1q = nullptr, *w2q = nullptr;
+  uint16_t *w1s = nullptr, *w2s = nullptr;
   float *rms_w = nullptr;  // weight of the RMS norm in front of the layer [H] (bf16 values), optional
   bool uploaded = false;
 };
@@ -81,8 +86,8 @@ hipError_t launch_pack_router(const float *w_src, const float *b_src, uint16_t *
                               int E, int E_pad, int H, hipStream_t s);
 hipError_t launch_pack_weight(const float *src, uint16_t *dst, int rows, int cols, bool gate_up,
                               hipStream_t s);
-hipError_t launch_pack_weight_mxfp4(const uint8_t *blocks, const uint8_t *scales, uint16_t *dst,
-                                    int rows, int cols, bool gate_up, hipStream_t s);
+hipError_t launch_pack_fp4(const uint8_t *blocks, const uint8_t *scales, uint8_t *wq, uint16_t *ws,
+                           int rows, int cols, bool gate_up, hipStream_t s);
 hipError_t launch_pack_bias(const float *src, float *dst_a, float *dst_b, int n, bool deinterleave,
                             hipStream_t s);
 
@@ -108,12 +113,12 @@ hipError_t launch_dispatch(const int *topk_i, const int *pos, int T, int E, int 
 hipError_t launch_gather(const uint16_t *x, const DispatchBuffers &d, uint16_t *xg, int T, int H,
                          int rb_cap, hipStream_t s);
 
-hipError_t launch_gate_up(const uint16_t *xg, const uint16_t *w1, const float *b1g, const float *b1u,
-                          const DispatchBuffers &d, uint16_t *act, int H, int IM, int E, float limit,
-                          int mt_cap, hipStream_t s);
-hipError_t launch_down(const uint16_t *act, const uint16_t *w2, const float *b2,
-                       const DispatchBuffers &d, float *y, int H, int IM, int E, int mt_cap,
-                       hipStream_t s);
+// w*_scale == nullptr: w* are bf16 fragments; otherwise MXFP4 chunks + scale bytes.
+hipError_t launch_gate_up(const uint16_t *xg, const void *w1, const uint16_t *w1_scale,
+                          const float *b1g, const float *b1u, const DispatchBuffers &d, uint16_t *act,
+                          int H, int IM, float limit, int mt_cap, hipStream_t s);
+hipError_t launch_down(const uint16_t *act, const void *w2, const uint16_t *w2_scale, const float *b2,
+                       const DispatchBuffers &d, float *y, int H, int IM, int mt_cap, hipStream_t s);
 hipError_t launch_combine(const float *y, const int *inv, const float *topk_v, const int *pos,
                           float *out, int T, int H, int accumulate, hipStream_t s);
 hipError_t launch_combine_residual(const float *y, const int *inv, const float *topk_v,

@@ -55,41 +55,43 @@ __global__ void pack_weight_kernel(const float *__restrict__ src, uint4 *__restr
 // MXFP4 ingest (export_model_bin/gpt-oss-20b/export_model_bin.py:86-123): a
 // row of `cols` weights is cols/32 blocks of 16 bytes plus one scale byte per
 // block; byte b of a block holds element 2b in its low nibble and element 2b+1
-// in its high nibble; a nibble indexes the table below and the scale byte s
-// multiplies by 2^(s - 127) (ldexp, as the exporter does).  Output: the same
-// bf16 fragments as pack_weight_kernel writes, so the GEMMs do not know the
-// difference.  The table values carry two significant bits, so the bf16 result
-// is exact wherever it is in range.
-__constant__ float kFp4Values[16] = {+0.0f, +0.5f, +1.0f, +1.5f, +2.0f, +3.0f, +4.0f, +6.0f,
-                                     -0.0f, -0.5f, -1.0f, -1.5f, -2.0f, -3.0f, -4.0f, -6.0f};
-
-__global__ void pack_weight_mxfp4_kernel(const uint8_t *__restrict__ blocks,
-                                         const uint8_t *__restrict__ scales, uint4 *__restrict__ dst,
-                                         int rows, int cols, int gate_up) {
-  const int kb_total = cols / kFragK;
-  const int groups = cols / 32;
-  const size_t n_chunks = (size_t)(rows / kRowBlock) * kb_total * 64;
+// in its high nibble; a nibble indexes {0, .5, 1, 1.5, 2, 3, 4, 6} and their
+// negatives, and the scale byte s multiplies by 2^(s - 127).  The weights stay
+// in this format on the device, re-ordered for the GEMMs that decode them in
+// registers (gemm_tile with FP4).  Per pair of row blocks (2P, 2P+1) and step of 32 k (one
+// MXFP4 block): a 16-byte chunk per lane l = (row n = l % 32, half h = l / 32),
+//   bytes 0-3   row of block 2P,   k block 0: elements 8h .. 8h+7  = source bytes 4h .. 4h+3
+//   bytes 4-7   row of block 2P,   k block 1: elements 16+8h ..    = source bytes 8+4h ..
+//   bytes 8-15  the same for block 2P+1,
+// and for every n the two scale bytes (block 2P, block 2P+1).  With gate_up set
+// the row blocks are the (gate, up) pairs of pack_weight_kernel.
+__global__ void pack_fp4_kernel(const uint8_t *__restrict__ blocks, const uint8_t *__restrict__ scales,
+                                uint4 *__restrict__ wq, uint16_t *__restrict__ ws, int rows, int cols,
+                                int gate_up) {
+  const int steps = cols / 32;
+  const int pairs = rows / (2 * kRowBlock);
+  const size_t n_chunks = (size_t)pairs * steps * 64;
   for (size_t c = (size_t)blockIdx.x * blockDim.x + threadIdx.x; c < n_chunks;
        c += (size_t)gridDim.x * blockDim.x) {
     const int lane = (int)(c & 63);
-    const size_t frag = c >> 6;
-    const int kb = (int)(frag % kb_total);
-    const int nb = (int)(frag / kb_total);
-    const int n = lane & 31;
-    const int k0 = kb * kFragK + 8 * (lane >> 5);  // 8 consecutive elements of one block
-    const int row = gate_up ? 2 * (kRowBlock * (nb >> 1) + n) + (nb & 1) : kRowBlock * nb + n;
-    const size_t g = (size_t)row * groups + k0 / 32;
-    const uint32_t bytes = *reinterpret_cast<const uint32_t *>(blocks + g * 16 + (k0 % 32) / 2);
-    const int expo = (int)scales[g] - 127;
+    const size_t ps = c >> 6;
+    const int step = (int)(ps % steps);
+    const int P = (int)(ps / steps);
+    const int n = lane & 31, h = lane >> 5;
     uint32_t o[4];
+    uint32_t sc = 0;
 #pragma unroll
-    for (int b = 0; b < 4; b++) {
-      const uint32_t byte = (bytes >> (8 * b)) & 0xffu;
-      const float lo = ldexpf(kFp4Values[byte & 15u], expo);
-      const float hi = ldexpf(kFp4Values[byte >> 4], expo);
-      o[b] = f32_to_bf16_rne(lo) | ((uint32_t)f32_to_bf16_rne(hi) << 16);
+    for (int j = 0; j < 2; j++) {
+      const int nb = 2 * P + j;
+      const int row = gate_up ? 2 * (kRowBlock * (nb >> 1) + n) + (nb & 1) : kRowBlock * nb + n;
+      const size_t g = (size_t)row * steps + step;
+      const uint8_t *src = blocks + g * 16;
+      o[2 * j + 0] = *reinterpret_cast<const uint32_t *>(src + 4 * h);
+      o[2 * j + 1] = *reinterpret_cast<const uint32_t *>(src + 8 + 4 * h);
+      sc |= (uint32_t)scales[g] << (8 * j);
     }
-    dst[c] = make_uint4(o[0], o[1], o[2], o[3]);
+    wq[c] = make_uint4(o[0], o[1], o[2], o[3]);
+    if (h == 0) ws[((size_t)P * steps + step) * 32 + n] = (uint16_t)sc;
   }
 }
 
@@ -147,10 +149,10 @@ hipError_t launch_pack_weight(const float *src, uint16_t *dst, int rows, int col
   return hipGetLastError();
 }
 
-hipError_t launch_pack_weight_mxfp4(const uint8_t *blocks, const uint8_t *scales, uint16_t *dst,
-                                    int rows, int cols, bool gate_up, hipStream_t s) {
-  pack_weight_mxfp4_kernel<<<2048, 256, 0, s>>>(blocks, scales, reinterpret_cast<uint4 *>(dst), rows,
-                                                cols, gate_up ? 1 : 0);
+hipError_t launch_pack_fp4(const uint8_t *blocks, const uint8_t *scales, uint8_t *wq, uint16_t *ws,
+                           int rows, int cols, bool gate_up, hipStream_t s) {
+  pack_fp4_kernel<<<2048, 256, 0, s>>>(blocks, scales, reinterpret_cast<uint4 *>(wq), ws, rows, cols,
+                                       gate_up ? 1 : 0);
   return hipGetLastError();
 }
 

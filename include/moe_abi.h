@@ -90,10 +90,13 @@ int moe_upload_layer(moe_handle *h, int layer, const float *w_router,
  * blocks is u8 [E, rows, cols/32, 16] and scales u8 [E, rows, cols/32]; byte b
  * of a block holds element 2b in its low and element 2b+1 in its high nibble, a
  * nibble indexes {0, .5, 1, 1.5, 2, 3, 4, 6, -0, -.5, -1, -1.5, -2, -3, -4, -6}
- * and the scale byte s multiplies by 2^(s-127).  Takes the place of
- * dequantize_fp4 in the exporter
+ * and the scale byte s multiplies by 2^(s-127) (s in 1..254).  Takes the place
+ * of dequantize_fp4 in the exporter
  * (export_model_bin/gpt-oss-20b/export_model_bin.py:66-123) followed by the fp32
- * upload; the decoded values are kept as bf16, which holds them exactly.
+ * upload.  The matrices stay MXFP4 in device memory (a quarter of the bytes of
+ * bf16); the GEMMs turn them into bf16 matrix-core operands in registers, which
+ * is exact, so the layer's results are those of an upload of the decoded
+ * matrices, bit for bit.
  * Router weights and all biases stay fp32 arguments.  Synchronous. */
 int moe_upload_layer_mxfp4(moe_handle *h, int layer, const float *w_router,
                            const float *b_router,

@@ -282,12 +282,13 @@ def test_c4_120b_shape():
 
 
 def test_c5_mxfp4_ingest():
-    """Expert matrices uploaded as MXFP4 blocks and scales.  The oracle decodes
-    them on the CPU (closed form pinned in tests/test_oracle.py); its values are
-    exact in bf16, so the GPU decode must lead to bit-identical outputs as an
-    upload of the decoded fp32 matrices, and the layer must match the oracle run
-    on those matrices.  Outputs are large here (weights up to 24), hence the
-    absolute bar scales with the output."""
+    """Expert matrices uploaded as MXFP4 blocks and scales: they stay MXFP4 on
+    the device and the GEMMs decode them in registers.  The oracle decodes them
+    on the CPU (closed form pinned in tests/test_oracle.py); its values are
+    exact in bf16, so the MXFP4 path must give bit-identical outputs to an
+    upload of the decoded fp32 matrices (the bf16 path), and the layer must
+    match the oracle run on those matrices.  Outputs are large here (weights up
+    to 24), hence the absolute bar scales with the output."""
     sh = synth.CONFIGS["c5"]
     x = synth.round_bf16(synth.make_activations(sh))
     wr, br = (synth.round_bf16(a) for a in synth.make_router(sh))
