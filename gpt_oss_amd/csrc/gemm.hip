@@ -183,11 +183,13 @@ __device__ __forceinline__ void gemm_tile(const uint4 *__restrict__ a_frag,  // 
   float4 bias_g[NBW / 2 + 1][4], bias_u[NBW / 2 + 1][4];
   float bias_d[NBW];
   if (GATE_UP) {
-    const int pairs_valid = max(1, (nb_valid - w * NBW) >> 1);
+    // a wave past the matrix's last column (last column tile only) reads the
+    // last valid pair's bias: the expert's bias vector ends there
+    const int P_last = ((nb0 + nb_valid) >> 1) - 1;
     const int P0 = (nb0 + w * NBW) >> 1;
 #pragma unroll
     for (int p = 0; p < NBW / 2; p++) {
-      const int P = P0 + min(p, pairs_valid - 1);
+      const int P = min(P0 + p, P_last);
 #pragma unroll
       for (int g = 0; g < 4; g++) {
         const int j = kRowBlock * P + 8 * g + 4 * (lane >> 5);
