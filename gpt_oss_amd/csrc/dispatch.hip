@@ -48,70 +48,71 @@ __global__ __launch_bounds__(kDispThreads) void dispatch_count_kernel(
     perm[i] = -1;
 }
 
-__device__ __forceinline__ int block_exclusive_scan_256(int v, int *buf, int tid, int *total) {
-  buf[tid] = v;
-  __syncthreads();
-#pragma unroll
-  for (int off = 1; off < 256; off <<= 1) {
-    const int add = tid >= off ? buf[tid - off] : 0;
-    __syncthreads();
-    buf[tid] += add;
-    __syncthreads();
-  }
-  const int incl = buf[tid];
-  *total = buf[255];
-  __syncthreads();
-  return incl - v;
-}
+// The plan of one batch from the experts' row counts (thread e holds expert e's
+// count; all 256 threads of the workgroup call this together).  Returns the
+// expert's first row in the padded row space.
+struct PlanOut {
+  int *offsets;
+  ExpertInfo *info;
+  int *totals;
+  TileDesc *tiles_gate_up, *tiles_down;
+  int tile_cap_gate_up, tile_cap_down;
+};
 
-// Pass 2 (one workgroup): turns the per-workgroup counts into exclusive bases,
-// and builds per-expert offsets and the row-tile plan of the grouped GEMMs.
-// An expert with M rows has ceil(M / 32) row blocks, cut into n_mt = ceil(row
-// blocks / 8) tiles as evenly as they go: the first `extra` tiles are rb + 1
-// row blocks high, the others rb.  Its segment in the padded row space is its
-// row blocks and no more, so an expert pads to at most 31 rows.
-//
-// It also cuts the tile sequence of either GEMM (n_ct column tiles per row
-// tile) into the 8 ranges of the XCDs, by estimated cost: a tile of r row blocks
-// costs kCostPerTile + kCostPerRowBlock * r.
-__global__ __launch_bounds__(256) void dispatch_scan_kernel(int *__restrict__ blk_counts, int n_blk,
-                                                           int E, int n_ct_gate_up, int n_ct_down,
-                                                           int *__restrict__ offsets,
-                                                           ExpertInfo *__restrict__ info,
-                                                           int *__restrict__ totals,
-                                                           TileDesc *__restrict__ tiles_gate_up,
-                                                           TileDesc *__restrict__ tiles_down,
-                                                           int tile_cap_gate_up, int tile_cap_down) {
-  __shared__ int buf[256];
+__device__ __forceinline__ int build_plan(int count, int E, int n_ct_gate_up, int n_ct_down,
+                                          const PlanOut &out, int *ex_count_out,
+                                          int *tot_count_out = nullptr) {
+  __shared__ int sh_wave[4][4];  // [wave][quantity]: the waves' sums
   __shared__ int sh_nmt[256], sh_rb[256], sh_extra[256], sh_rowblk[256];
   __shared__ int sh_cost[257];   // exclusive prefix of the experts' cost per column tile
   __shared__ int sh_tiles[257];  // exclusive prefix of their row tiles
   __shared__ int sh_bound[2][kXcds + 1];
   const int e = threadIdx.x;
-  int count = 0;
-  if (e < E) {
-    // 16 independent loads at a time, then their running sums back in place
-    for (int b0 = 0; b0 < n_blk; b0 += 16) {
-      int c[16];
-#pragma unroll
-      for (int i = 0; i < 16; i++) c[i] = b0 + i < n_blk ? blk_counts[(size_t)(b0 + i) * E + e] : 0;
-#pragma unroll
-      for (int i = 0; i < 16; i++) {
-        if (b0 + i < n_blk) blk_counts[(size_t)(b0 + i) * E + e] = count;
-        count += c[i];
-      }
-    }
-  }
+  const int lane = e & 63;
+  const int w = e >> 6;
+  int *offsets = out.offsets;
+  ExpertInfo *info = out.info;
+  int *totals = out.totals;
   const int n_rb = (count + kRowBlock - 1) / kRowBlock;
   constexpr int kTileRb = kTileRows / kRowBlock;
   const int n_mt = (n_rb + kTileRb - 1) / kTileRb;
   const int rb = n_mt ? n_rb / n_mt : 0;
   const int extra = n_mt ? n_rb - rb * n_mt : 0;
-  const int padded = n_rb * kRowBlock;
-  int tot_count, tot_pad, tot_mt;
-  const int ex_count = block_exclusive_scan_256(count, buf, e, &tot_count);
-  const int ex_pad = block_exclusive_scan_256(padded, buf, e, &tot_pad);
-  const int ex_mt = block_exclusive_scan_256(n_mt, buf, e, &tot_mt);
+  // cost of one column tile's worth of the expert's row tiles
+  const int cost = n_mt * (kCostPerTile + kCostPerRowBlock * rb) + kCostPerRowBlock * extra;
+  // Exclusive prefix sums over the experts of four quantities at once: rows,
+  // padded rows, row tiles, cost.  In a wave by lane shifts, across the four
+  // waves through LDS.
+  const int own[4] = {count, n_rb * kRowBlock, n_mt, cost};
+  int incl[4] = {own[0], own[1], own[2], own[3]};
+#pragma unroll
+  for (int off = 1; off < 64; off <<= 1) {
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      const int up = __shfl_up(incl[i], off, 64);
+      if (lane >= off) incl[i] += up;
+    }
+  }
+  if (lane == 63) {
+#pragma unroll
+    for (int i = 0; i < 4; i++) sh_wave[w][i] = incl[i];
+  }
+  __syncthreads();
+  int ex[4], tot[4];
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    int below = 0, all = 0;
+#pragma unroll
+    for (int ww = 0; ww < 4; ww++) {
+      const int v = sh_wave[ww][i];
+      below += ww < w ? v : 0;
+      all += v;
+    }
+    ex[i] = below + incl[i] - own[i];
+    tot[i] = all;
+  }
+  const int ex_count = ex[0], ex_pad = ex[1], ex_mt = ex[2], ex_cost = ex[3];
+  const int tot_count = tot[0], tot_pad = tot[1], tot_mt = tot[2], tot_cost = tot[3];
   if (e < E) {
     offsets[e] = ex_count;
     ExpertInfo inf;
@@ -124,10 +125,6 @@ __global__ __launch_bounds__(256) void dispatch_scan_kernel(int *__restrict__ bl
     inf.pad_[0] = inf.pad_[1] = 0;
     info[e] = inf;
   }
-  // cost of one column tile's worth of the expert's row tiles
-  const int cost = n_mt * (kCostPerTile + kCostPerRowBlock * rb) + kCostPerRowBlock * extra;
-  int tot_cost;
-  const int ex_cost = block_exclusive_scan_256(cost, buf, e, &tot_cost);
   sh_cost[e] = ex_cost;
   sh_tiles[e] = ex_mt;
   sh_nmt[e] = n_mt;
@@ -175,47 +172,83 @@ __global__ __launch_bounds__(256) void dispatch_scan_kernel(int *__restrict__ bl
     }
     sh_bound[g][x] = bound;
   }
+  // The tile sequences: tile L = (expert, column tile, row tile), row tile
+  // fastest.  The waves take the experts in turn, the lanes the expert's tiles.
+  for (int ee = w; ee < E; ee += 4) {
+    const int nmt = sh_nmt[ee];
+    if (nmt == 0) continue;
+    const int rbe = sh_rb[ee], exe = sh_extra[ee], rowblk = sh_rowblk[ee], first = sh_tiles[ee];
+    for (int g = 0; g < 2; g++) {
+      const int n_ct = g ? n_ct_down : n_ct_gate_up;
+      TileDesc *tiles = g ? out.tiles_down : out.tiles_gate_up;
+      const int cap = g ? out.tile_cap_down : out.tile_cap_gate_up;
+      const int n = nmt * n_ct;
+      for (int i = lane; i < n; i += 64) {
+        const int L = first * n_ct + i;
+        const int nt = i / nmt;
+        const int mt = i - nt * nmt;
+        TileDesc d;
+        d.e = ee;
+        d.nt = nt;
+        d.rbt = rbe + (mt < exe ? 1 : 0);
+        d.rb0 = rowblk + mt * rbe + min(mt, exe);
+        if (L < cap) tiles[L] = d;
+      }
+    }
+  }
   __syncthreads();
   // keep every range within what the launch grid provides for (xcd_tile_cap)
   if (e < 2) {
     const int n_ct = e ? n_ct_down : n_ct_gate_up;
     const int total_tiles = tot_mt * n_ct;
     const int cap = xcd_tile_cap(total_tiles);
-    int *out = totals + (e ? kTotBoundsDown : kTotBoundsGateUp);
+    int *bounds = totals + (e ? kTotBoundsDown : kTotBoundsGateUp);
     int prev = 0;
-    out[0] = 0;
+    bounds[0] = 0;
     for (int x = 1; x < kXcds; x++) {
       int bnd = sh_bound[e][x];
       bnd = max(bnd, max(prev, total_tiles - (kXcds - x) * cap));
       bnd = min(bnd, prev + cap);
-      out[x] = bnd;
+      bounds[x] = bnd;
       prev = bnd;
     }
-    out[kXcds] = total_tiles;
+    bounds[kXcds] = total_tiles;
   }
-  // The tile sequences: tile L = (expert, column tile, row tile), row tile fastest.
-  for (int g = 0; g < 2; g++) {
-    const int n_ct = g ? n_ct_down : n_ct_gate_up;
-    TileDesc *tiles = g ? tiles_down : tiles_gate_up;
-    const int total_tiles = min(tot_mt * n_ct, g ? tile_cap_down : tile_cap_gate_up);
-    for (int L = e; L < total_tiles; L += 256) {
-      // last expert whose first tile is at or before L; experts without rows share
-      // their successor's start and are passed over
-      int lo = 0, hi = 255;
-      while (lo < hi) {
-        const int mid = (lo + hi + 1) >> 1;
-        if (sh_tiles[mid] * n_ct <= L) lo = mid; else hi = mid - 1;
+  *ex_count_out = ex_count;
+  if (tot_count_out) *tot_count_out = tot_count;
+  return ex_pad;
+}
+
+// Pass 2 (one workgroup): turns the per-workgroup counts into exclusive bases,
+// and builds per-expert offsets and the row-tile plan of the grouped GEMMs.
+// An expert with M rows has ceil(M / 32) row blocks, cut into n_mt = ceil(row
+// blocks / 8) tiles as evenly as they go: the first `extra` tiles are rb + 1
+// row blocks high, the others rb.  Its segment in the padded row space is its
+// row blocks and no more, so an expert pads to at most 31 rows.
+//
+// It also cuts the tile sequence of either GEMM (n_ct column tiles per row
+// tile) into the 8 ranges of the XCDs, by estimated cost: a tile of r row blocks
+// costs kCostPerTile + kCostPerRowBlock * r.
+__global__ __launch_bounds__(256) void dispatch_scan_kernel(int *__restrict__ blk_counts, int n_blk,
+                                                           int E, int n_ct_gate_up, int n_ct_down,
+                                                           PlanOut out) {
+  const int e = threadIdx.x;
+  int count = 0;
+  if (e < E) {
+    // 16 independent loads at a time, then their running sums back in place
+    for (int b0 = 0; b0 < n_blk; b0 += 16) {
+      int c[16];
+#pragma unroll
+      for (int i = 0; i < 16; i++) c[i] = b0 + i < n_blk ? blk_counts[(size_t)(b0 + i) * E + e] : 0;
+#pragma unroll
+      for (int i = 0; i < 16; i++) {
+        if (b0 + i < n_blk) blk_counts[(size_t)(b0 + i) * E + e] = count;
+        count += c[i];
       }
-      const int rem = L - sh_tiles[lo] * n_ct;
-      const int mt = rem % sh_nmt[lo];
-      TileDesc d;
-      d.e = lo;
-      d.nt = rem / sh_nmt[lo];
-      d.rbt = sh_rb[lo] + (mt < sh_extra[lo] ? 1 : 0);
-      d.rb0 = sh_rowblk[lo] + mt * sh_rb[lo] + min(mt, sh_extra[lo]);
-      tiles[L] = d;
     }
   }
+  int ex_count;
+  build_plan(count, E, n_ct_gate_up, n_ct_down, out, &ex_count);
 }
 
 // Pass 3: rank of every assignment inside its expert = (assignments of lower
@@ -276,6 +309,107 @@ __global__ __launch_bounds__(kDispThreads) void dispatch_scatter_kernel(
   }
   *reinterpret_cast<int4 *>(inv + (size_t)t * kTopK) =
       make_int4(out_inv[0], out_inv[1], out_inv[2], out_inv[3]);
+}
+
+// Passes 1-3 in one workgroup for batches of at most kSmallRounds x 256 tokens:
+// the rounds of 256 tokens play the part of the workgroups of the three-kernel
+// form (round r's assignments come after those of the rounds before it), so
+// the result is the same, bit for bit.
+constexpr int kSmallRounds = 2;
+
+__global__ __launch_bounds__(kDispThreads) void dispatch_small_kernel(
+    const int *__restrict__ topk_i, const int *__restrict__ pos, int T, int E, int n_ct_gate_up,
+    int n_ct_down, PlanOut out, int *__restrict__ perm, int *__restrict__ rowmap,
+    int *__restrict__ inv) {
+  __shared__ int hist[kSmallRounds][256];  // per round and expert: count, then exclusive base
+  __shared__ int sh_off[256], sh_row0[256];
+  __shared__ int wave_cnt[kDispThreads / 64][256];
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int w = tid >> 6;
+  const int n_round = (T + kDispThreads - 1) / kDispThreads;
+#pragma unroll
+  for (int r = 0; r < kSmallRounds; r++) hist[r][tid] = 0;
+  __syncthreads();
+  int id[kSmallRounds][kTopK];
+#pragma unroll
+  for (int r = 0; r < kSmallRounds; r++) {
+    const int t = r * kDispThreads + tid;
+#pragma unroll
+    for (int k = 0; k < kTopK; k++) id[r][k] = -1;
+    if (r < n_round && t < T && !(pos && pos[t] < 0)) {
+      const int4 ids = *reinterpret_cast<const int4 *>(topk_i + (size_t)t * kTopK);
+      id[r][0] = ids.x; id[r][1] = ids.y; id[r][2] = ids.z; id[r][3] = ids.w;
+#pragma unroll
+      for (int k = 0; k < kTopK; k++) {
+        if (id[r][k] < 0 || id[r][k] >= E) id[r][k] = -1;
+        if (id[r][k] >= 0) atomicAdd(&hist[r][id[r][k]], 1);
+      }
+    }
+  }
+  __syncthreads();
+  // expert tid: counts of the rounds -> exclusive bases, total -> plan
+  int count = 0;
+#pragma unroll
+  for (int r = 0; r < kSmallRounds; r++) {
+    const int c = hist[r][tid];
+    hist[r][tid] = count;
+    count += c;
+  }
+  int ex_count, tot_count;
+  const int row0 = build_plan(tid < E ? count : 0, E, n_ct_gate_up, n_ct_down, out, &ex_count, &tot_count);
+  sh_off[tid] = ex_count;
+  sh_row0[tid] = row0;
+  // -1 where the scatter below writes nothing: the padding rows of the experts
+  // and the tail of perm that inactive rows and invalid ids leave unused
+  if (tid < E) {
+    const int end = row0 + (count + kRowBlock - 1) / kRowBlock * kRowBlock;
+    for (int i = row0 + count; i < end; i++) rowmap[i] = -1;
+  }
+  for (int i = tot_count + tid; i < T * kTopK; i += kDispThreads) perm[i] = -1;
+  __syncthreads();
+  // stable ranks, as dispatch_scatter_kernel
+  const unsigned long long lt = (1ull << lane) - 1ull;
+#pragma unroll
+  for (int r = 0; r < kSmallRounds; r++) {
+    if (r >= n_round) break;
+    int rank[kTopK] = {0, 0, 0, 0};
+    for (int e = 0; e < E; e++) {
+      int below = 0, total = 0, mine = 0;
+#pragma unroll
+      for (int k = 0; k < kTopK; k++) {
+        const bool hit = id[r][k] == e;
+        const unsigned long long m = __ballot(hit);
+        below += __popcll(m & lt);
+        total += __popcll(m);
+        if (hit) rank[k] = mine;
+        mine += hit ? 1 : 0;
+      }
+#pragma unroll
+      for (int k = 0; k < kTopK; k++)
+        if (id[r][k] == e) rank[k] += below;
+      if (lane == 0) wave_cnt[w][e] = total;
+    }
+    __syncthreads();
+    const int t = r * kDispThreads + tid;
+    if (t < T) {
+      int out_inv[kTopK];
+#pragma unroll
+      for (int k = 0; k < kTopK; k++) {
+        const int e = id[r][k];
+        if (e < 0) { out_inv[k] = -1; continue; }
+        int rk = hist[r][e] + rank[k];
+        for (int ww = 0; ww < w; ww++) rk += wave_cnt[ww][e];
+        const int prow = sh_row0[e] + rk;
+        perm[sh_off[e] + rk] = t * kTopK + k;
+        rowmap[prow] = t * kTopK + k;
+        out_inv[k] = prow;
+      }
+      *reinterpret_cast<int4 *>(inv + (size_t)t * kTopK) =
+          make_int4(out_inv[0], out_inv[1], out_inv[2], out_inv[3]);
+    }
+    __syncthreads();  // wave_cnt is reused by the next round
+  }
 }
 
 // Copies the routed rows of x into the padded per-expert row space, already in
@@ -361,11 +495,23 @@ hipError_t launch_dispatch(const int *topk_i, const int *pos, int T, int E, int 
   const long long A = (long long)T * kTopK;
   const long long reach = A + (long long)kTileGran * E;
   const int fill_rows = (int)(reach < d.a_pad_cap ? reach : d.a_pad_cap);
+  PlanOut plan;
+  plan.offsets = d.offsets;
+  plan.info = d.info;
+  plan.totals = d.totals;
+  plan.tiles_gate_up = d.tiles_gate_up;
+  plan.tiles_down = d.tiles_down;
+  plan.tile_cap_gate_up = d.tile_cap_gate_up;
+  plan.tile_cap_down = d.tile_cap_down;
+  if (n_blk <= kSmallRounds) {
+    // small batches: one workgroup does all three passes, two launches fewer
+    dispatch_small_kernel<<<1, kDispThreads, 0, s>>>(topk_i, pos, T, E, n_ct_gate_up, n_ct_down, plan,
+                                                     d.perm, d.rowmap, d.inv);
+    return hipGetLastError();
+  }
   dispatch_count_kernel<<<n_blk, kDispThreads, 0, s>>>(topk_i, pos, T, E, d.blk_counts, d.rowmap,
                                                        fill_rows, d.perm);
-  dispatch_scan_kernel<<<1, 256, 0, s>>>(d.blk_counts, n_blk, E, n_ct_gate_up, n_ct_down, d.offsets,
-                                         d.info, d.totals, d.tiles_gate_up, d.tiles_down,
-                                         d.tile_cap_gate_up, d.tile_cap_down);
+  dispatch_scan_kernel<<<1, 256, 0, s>>>(d.blk_counts, n_blk, E, n_ct_gate_up, n_ct_down, plan);
   dispatch_scatter_kernel<<<n_blk, kDispThreads, 0, s>>>(topk_i, pos, T, E, d.blk_counts, d.offsets,
                                                          d.info, d.perm, d.rowmap, d.inv);
   return hipGetLastError();

@@ -113,12 +113,15 @@ struct StageRing {
 
 // NW waves side by side over the columns, NBW column blocks per wave, R ring
 // slots (LDS stages for the row operand, register slots for the column operand).
-template <int NW_, int NBW_, int R_>
+// RBM = row blocks per tile at most: it sizes the LDS stages, and with them how
+// many workgroups share a CU; WAVES = waves per SIMD the registers are held to.
+template <int NW_, int NBW_, int R_, int RBM_ = kTileRows / kRowBlock, int WAVES_ = 1>
 struct GemmCfg {
   static constexpr int NW = NW_, NBW = NBW_, R = R_, KPS = 2;
   static constexpr int THREADS = NW * 64;
+  static constexpr int WAVES = WAVES_;
   static constexpr int TILE_NB = NW * NBW;              // column blocks per tile
-  static constexpr int RBT_MAX = kTileRows / kRowBlock;  // row blocks per tile, at most
+  static constexpr int RBT_MAX = RBM_;                   // row blocks per tile, at most
   static constexpr int STAGE = RBT_MAX * KPS * 64;       // uint4 per LDS stage (16 KB)
   static constexpr int EPI_LD = NBW * 32 + 8;            // floats per buffered output row
   static constexpr int EPI_WAVE = 32 * EPI_LD / 4;       // uint4 per wave of epilogue buffer
@@ -477,7 +480,7 @@ __device__ __forceinline__ void gemm_tile(const uint4 *__restrict__ a_frag,  // 
 }
 
 template <typename C, bool GATE_UP, bool FP4>
-__global__ __launch_bounds__(C::THREADS) void grouped_gemm_kernel(
+__global__ __launch_bounds__(C::THREADS, C::WAVES) void grouped_gemm_kernel(
     const uint4 *__restrict__ a_frag, const uint4 *__restrict__ w_frag,
     const uint16_t *__restrict__ w_scale,
     const float *__restrict__ bias_a, const float *__restrict__ bias_b,
@@ -500,14 +503,24 @@ __global__ __launch_bounds__(C::THREADS) void grouped_gemm_kernel(
   const uint16_t *b_scale = FP4 ? w_scale + (size_t)tc.e * nb_total * KB * 8 : nullptr;
   const float *ba = bias_a + (size_t)tc.e * N;
   const float *bb = GATE_UP ? bias_b + (size_t)tc.e * N : nullptr;
-#define MOE_TILE_CASE(n) \
-  case n: gemm_tile<n, C, GATE_UP, FP4>(a_frag, b_frag, b_scale, KB, tc.rb0, nb0, nb_valid, ba, bb, outp, N, limit, st0, st1, st2, st3, st4, st5, st6, epi); break;
-  switch (tc.rbt) {
-    MOE_TILE_CASE(1) MOE_TILE_CASE(2) MOE_TILE_CASE(3) MOE_TILE_CASE(4)
-    MOE_TILE_CASE(5) MOE_TILE_CASE(6) MOE_TILE_CASE(7)
-    default: gemm_tile<8, C, GATE_UP, FP4>(a_frag, b_frag, b_scale, KB, tc.rb0, nb0, nb_valid, ba, bb, outp, N, limit, st0, st1, st2, st3, st4, st5, st6, epi); break;
+#define MOE_TILE(n) \
+  gemm_tile<n, C, GATE_UP, FP4>(a_frag, b_frag, b_scale, KB, tc.rb0, nb0, nb_valid, ba, bb, outp, N, limit, st0, st1, st2, st3, st4, st5, st6, epi)
+  if constexpr (C::RBT_MAX == 8) {
+    switch (tc.rbt) {
+      case 1: MOE_TILE(1); break;
+      case 2: MOE_TILE(2); break;
+      case 3: MOE_TILE(3); break;
+      case 4: MOE_TILE(4); break;
+      case 5: MOE_TILE(5); break;
+      case 6: MOE_TILE(6); break;
+      case 7: MOE_TILE(7); break;
+      default: MOE_TILE(8); break;
+    }
+  } else {
+    static_assert(C::RBT_MAX == 2, "tile heights of the small-batch configuration");
+    if (tc.rbt == 1) MOE_TILE(1); else MOE_TILE(2);
   }
-#undef MOE_TILE_CASE
+#undef MOE_TILE
 }
 
 // 4 waves, one per SIMD, each 256 rows x 64 columns (8 x 2 accumulators = all
@@ -515,6 +528,13 @@ __global__ __launch_bounds__(C::THREADS) void grouped_gemm_kernel(
 using CfgGemm = GemmCfg<4, 2, 7>;
 static_assert(CfgGemm::RBT_MAX * kRowBlock == kTileRows && CfgGemm::TILE_NB == kGemmTileNb,
               "tile plan of dispatch_scan_kernel");
+// Batches of at most 64 tokens: no expert has more than 64 rows, every tile is
+// one or two row blocks high and the GEMMs are a stream of weights.  What
+// limits that stream is the bytes one CU keeps in flight, so the same kernel is
+// built with LDS stages for two row blocks and registers for two waves per
+// SIMD, and several workgroups share a CU.
+using CfgGemmSmall = GemmCfg<4, 2, 7, 2, 2>;
+constexpr int kSmallBatchTokens = CfgGemmSmall::RBT_MAX * kRowBlock;
 
 // w_scale == nullptr: w holds bf16 fragments; otherwise w holds MXFP4 chunks and
 // w_scale their scale bytes (pack_fp4_kernel).
@@ -538,14 +558,23 @@ static hipError_t launch_gemm(const uint4 *a, const uint4 *w, const uint16_t *w_
 
 hipError_t launch_gate_up(const uint16_t *xg, const void *w1, const uint16_t *w1_scale,
                           const float *b1g, const float *b1u, const DispatchBuffers &d, uint16_t *act,
-                          int H, int IM, float limit, int mt_cap, hipStream_t s) {
+                          int H, int IM, float limit, int mt_cap, int max_rows, hipStream_t s) {
+  if (max_rows <= kSmallBatchTokens)
+    return launch_gemm<CfgGemmSmall, true>(reinterpret_cast<const uint4 *>(xg),
+                                           reinterpret_cast<const uint4 *>(w1), w1_scale, b1g, b1u, d,
+                                           act, H, IM, limit, mt_cap, s);
   return launch_gemm<CfgGemm, true>(reinterpret_cast<const uint4 *>(xg),
                                     reinterpret_cast<const uint4 *>(w1), w1_scale, b1g, b1u, d, act, H,
                                     IM, limit, mt_cap, s);
 }
 
 hipError_t launch_down(const uint16_t *act, const void *w2, const uint16_t *w2_scale, const float *b2,
-                       const DispatchBuffers &d, float *y, int H, int IM, int mt_cap, hipStream_t s) {
+                       const DispatchBuffers &d, float *y, int H, int IM, int mt_cap, int max_rows,
+                       hipStream_t s) {
+  if (max_rows <= kSmallBatchTokens)
+    return launch_gemm<CfgGemmSmall, false>(reinterpret_cast<const uint4 *>(act),
+                                            reinterpret_cast<const uint4 *>(w2), w2_scale, b2, nullptr,
+                                            d, y, IM, H, 0.f, mt_cap, s);
   return launch_gemm<CfgGemm, false>(reinterpret_cast<const uint4 *>(act),
                                      reinterpret_cast<const uint4 *>(w2), w2_scale, b2, nullptr, d, y,
                                      IM, H, 0.f, mt_cap, s);

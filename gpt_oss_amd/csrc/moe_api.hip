@@ -126,8 +126,9 @@ inline int down_col_tiles(const moe_config &c) {
 }
 
 // out != nullptr: out (+)= layer(x), fp32.  Otherwise resid (bf16, in place) += layer(x).
+// max_rows: no expert is given more rows than this (T when the ids of a token are distinct).
 int run_experts(moe_handle *h, int layer, const uint16_t *x, const int *pos, const int *topk_i,
-                const float *topk_v, int T, float *out, int accumulate, hipStream_t s,
+                const float *topk_v, int T, int max_rows, float *out, int accumulate, hipStream_t s,
                 StageTimer &tm, uint16_t *resid = nullptr) {
   const moe_config &c = h->cfg;
   const LayerWeights &lw = h->layers[layer];
@@ -140,10 +141,10 @@ int run_experts(moe_handle *h, int layer, const uint16_t *x, const int *pos, con
   HIP_TRY(launch_gather(x, h->disp, h->xg, T, c.hidden, rb_cap, s));
   HIP_TRY(tm.mark(MOE_STAGE_GATE_UP));
   HIP_TRY(launch_gate_up(h->xg, lw.w1q ? static_cast<const void *>(lw.w1q) : lw.w1, lw.w1s, lw.b1g,
-                         lw.b1u, h->disp, h->act, c.hidden, c.inter, c.swiglu_limit, mt_cap, s));
+                         lw.b1u, h->disp, h->act, c.hidden, c.inter, c.swiglu_limit, mt_cap, max_rows, s));
   HIP_TRY(tm.mark(MOE_STAGE_DOWN));
   HIP_TRY(launch_down(h->act, lw.w2q ? static_cast<const void *>(lw.w2q) : lw.w2, lw.w2s, lw.b2,
-                      h->disp, h->y, c.hidden, c.inter, mt_cap, s));
+                      h->disp, h->y, c.hidden, c.inter, mt_cap, max_rows, s));
   HIP_TRY(tm.mark(MOE_STAGE_COMBINE));
   if (out) {
     HIP_TRY(launch_combine(h->y, h->disp.inv, topk_v, pos, out, T, c.hidden, accumulate, s));
@@ -435,7 +436,8 @@ int moe_experts(moe_handle *h, int layer, const uint16_t *x, const int *pos, con
   hipStream_t s = static_cast<hipStream_t>(stream);
   StageTimer tm(h, s);
   HIP_TRY(tm.mark(MOE_STAGE_ROUTER));
-  rc = run_experts(h, layer, x, pos, topk_i, topk_v, n_tokens, out, accumulate, s, tm);
+  // ids from outside may name an expert in several slots of a token
+  rc = run_experts(h, layer, x, pos, topk_i, topk_v, n_tokens, n_tokens * kTopK, out, accumulate, s, tm);
   if (rc == MOE_OK) tm.done();
   return rc;
 }
@@ -451,7 +453,7 @@ int moe_forward(moe_handle *h, int layer, const uint16_t *x, const int *pos, int
   HIP_TRY(tm.mark(MOE_STAGE_ROUTER));
   HIP_TRY(launch_router(x, pos, lw.wr, lw.br, n_tokens, h->cfg.hidden, h->cfg.experts, h->E_pad,
                         nullptr, h->topk_i, h->topk_v, s));
-  rc = run_experts(h, layer, x, pos, h->topk_i, h->topk_v, n_tokens, out, accumulate, s, tm);
+  rc = run_experts(h, layer, x, pos, h->topk_i, h->topk_v, n_tokens, n_tokens, out, accumulate, s, tm);
   if (rc == MOE_OK) tm.done();
   return rc;
 }
@@ -493,7 +495,8 @@ int moe_block_forward(moe_handle *h, int layer, uint16_t *x, const int *pos, int
   HIP_TRY(launch_rmsnorm(x, lw.rms_w, pos, h->t_norm, n_tokens, h->cfg.hidden, s));
   HIP_TRY(launch_router(h->t_norm, pos, lw.wr, lw.br, n_tokens, h->cfg.hidden, h->cfg.experts,
                         h->E_pad, nullptr, h->topk_i, h->topk_v, s));
-  rc = run_experts(h, layer, h->t_norm, pos, h->topk_i, h->topk_v, n_tokens, nullptr, 0, s, tm, x);
+  rc = run_experts(h, layer, h->t_norm, pos, h->topk_i, h->topk_v, n_tokens, n_tokens, nullptr, 0, s, tm,
+                   x);
   if (rc == MOE_OK) tm.done();
   return rc;
 }

@@ -116,9 +116,10 @@ hipError_t launch_gather(const uint16_t *x, const DispatchBuffers &d, uint16_t *
 // w*_scale == nullptr: w* are bf16 fragments; otherwise MXFP4 chunks + scale bytes.
 hipError_t launch_gate_up(const uint16_t *xg, const void *w1, const uint16_t *w1_scale,
                           const float *b1g, const float *b1u, const DispatchBuffers &d, uint16_t *act,
-                          int H, int IM, float limit, int mt_cap, hipStream_t s);
+                          int H, int IM, float limit, int mt_cap, int max_rows, hipStream_t s);
 hipError_t launch_down(const uint16_t *act, const void *w2, const uint16_t *w2_scale, const float *b2,
-                       const DispatchBuffers &d, float *y, int H, int IM, int mt_cap, hipStream_t s);
+                       const DispatchBuffers &d, float *y, int H, int IM, int mt_cap, int max_rows,
+                       hipStream_t s);
 hipError_t launch_combine(const float *y, const int *inv, const float *topk_v, const int *pos,
                           float *out, int T, int H, int accumulate, hipStream_t s);
 hipError_t launch_combine_residual(const float *y, const int *inv, const float *topk_v,

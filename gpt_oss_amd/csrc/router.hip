@@ -32,7 +32,7 @@ __device__ __forceinline__ void widen8(const uint4 v, double (&d)[8]) {
 // dimension in chunks of 32 (wave w takes chunks w, w+WPC, ...), each wave
 // keeps NT 16x16 accumulators, and the partial sums are added in wave order
 // through LDS.  NT = E_pad / 16.
-template <int NT, int WPC>
+template <int NT, int WPC, int D>
 __global__ __launch_bounds__(WPC * 64) void router_kernel(
     const uint16_t *__restrict__ x, const int *__restrict__ pos, const uint16_t *__restrict__ wr,
     const float *__restrict__ br, int T, int H, int E, float *__restrict__ score,
@@ -54,43 +54,46 @@ __global__ __launch_bounds__(WPC * 64) void router_kernel(
 #pragma unroll
   for (int n = 0; n < NT; n++) acc[n] = f64x4{0.0, 0.0, 0.0, 0.0};
 
-  // The loads of chunk c + WPC are issued before the MFMAs of chunk c: with few
-  // waves per SIMD nothing else would cover their latency.
+  // The wave's loads run D chunks ahead of its MFMAs (a ring of D register
+  // sets): with few waves per SIMD nothing else covers their latency, and a
+  // small batch is a handful of workgroups whose time is the chain of these
+  // round trips.  Past the end the ring re-loads the last chunk and drops it.
   const uint16_t *xrow = x + (size_t)t_ld * H + g * 8;
   const uint16_t *wlane = wr + (size_t)lane * 8;
-  uint4 xv = make_uint4(0, 0, 0, 0), wv[NT];
-  if (w < kc_total) {
-    xv = *reinterpret_cast<const uint4 *>(xrow + w * 32);
+  uint4 xs[D], ws[D][NT];
+  auto load = [&](int d, int c) {
+    const int cc = min(c, kc_total - 1);
+    xs[d] = *reinterpret_cast<const uint4 *>(xrow + cc * 32);
 #pragma unroll
     for (int n = 0; n < NT; n++)
-      wv[n] = *reinterpret_cast<const uint4 *>(wlane + ((size_t)n * kc_total + w) * 512);
-  }
-  for (int c = w; c < kc_total; c += WPC) {
-    const int cn = min(c + WPC, kc_total - 1);  // the last prefetch repeats a chunk and is dropped
-    const uint4 xn = *reinterpret_cast<const uint4 *>(xrow + cn * 32);
-    uint4 wn[NT];
+      ws[d][n] = *reinterpret_cast<const uint4 *>(wlane + ((size_t)n * kc_total + cc) * 512);
+  };
 #pragma unroll
-    for (int n = 0; n < NT; n++)
-      wn[n] = *reinterpret_cast<const uint4 *>(wlane + ((size_t)n * kc_total + cn) * 512);
-    double xd[8];
-    widen8(xv, xd);
-    // Two accumulators are advanced alternately so that back-to-back MFMAs do
-    // not depend on each other.
-    constexpr int NP = NT > 1 ? 2 : 1;
+  for (int d = 0; d < D; d++) load(d, w + d * WPC);
+  for (int c0 = w; c0 < kc_total; c0 += D * WPC) {
 #pragma unroll
-    for (int n = 0; n < NT; n += NP) {
-      double wd[NP][8];
+    for (int d = 0; d < D; d++) {
+      const int c = c0 + d * WPC;
+      if (c < kc_total) {  // the same for the whole wave
+        double xd[8];
+        widen8(xs[d], xd);
+        // Two accumulators are advanced alternately so that back-to-back MFMAs do
+        // not depend on each other.
+        constexpr int NP = NT > 1 ? 2 : 1;
 #pragma unroll
-      for (int p = 0; p < NP; p++) widen8(wv[n + p], wd[p]);
+        for (int n = 0; n < NT; n += NP) {
+          double wd[NP][8];
 #pragma unroll
-      for (int s = 0; s < 8; s++)
+          for (int p = 0; p < NP; p++) widen8(ws[d][n + p], wd[p]);
 #pragma unroll
-        for (int p = 0; p < NP; p++)
-          acc[n + p] = __builtin_amdgcn_mfma_f64_16x16x4f64(xd[s], wd[p][s], acc[n + p], 0, 0, 0);
+          for (int s = 0; s < 8; s++)
+#pragma unroll
+            for (int p = 0; p < NP; p++)
+              acc[n + p] = __builtin_amdgcn_mfma_f64_16x16x4f64(xd[s], wd[p][s], acc[n + p], 0, 0, 0);
+        }
+        load(d, c + D * WPC);
+      }
     }
-    xv = xn;
-#pragma unroll
-    for (int n = 0; n < NT; n++) wv[n] = wn[n];
   }
 
 #pragma unroll
@@ -185,7 +188,10 @@ static hipError_t launch_router_nt(const uint16_t *x, const int *pos, const uint
   // LDS for the partial sums allows (WPC * NT * 2 KB <= 64 KB): more waves per
   // SIMD hide the load latency, and small batches still occupy the SIMDs.
   constexpr int WPC = NT <= 2 ? 16 : (NT <= 4 ? 8 : (NT <= 8 ? 4 : 2));
-  router_kernel<NT, WPC><<<grid, WPC * 64, 0, s>>>(x, pos, wr, br, T, H, E, score, topk_i, topk_v);
+  // Register sets in flight per wave, 4 * (1 + NT) registers each, within the
+  // 128 / 256 / 512 registers a wave of a workgroup this size can have.
+  constexpr int D = NT <= 2 ? 6 : (NT <= 4 ? 4 : (NT <= 8 ? 3 : 2));
+  router_kernel<NT, WPC, D><<<grid, WPC * 64, 0, s>>>(x, pos, wr, br, T, H, E, score, topk_i, topk_v);
   return hipGetLastError();
 }
 
