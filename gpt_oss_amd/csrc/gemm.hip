@@ -69,6 +69,13 @@ __device__ __forceinline__ uint32_t pack_bf16(float a, float b) {
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
+// Row split of a column tile with nb_valid of its NW * NBW column blocks inside
+// the matrix: 4 when a quarter of the waves have columns, 2 when half have.
+__host__ __device__ inline int row_split_of(int nb_valid, int nw, int nbw) {
+  const int waves = (nb_valid + nbw - 1) / nbw;
+  return (nw == 4 && waves == 1) ? 4 : ((nw == 4 && waves == 2) ? 2 : 1);
+}
+
 // Maps the workgroup id to a tile (see "Tile order" above): two dependent
 // loads, the XCD's range and the tile's descriptor.  Returns false for the
 // surplus workgroups of the upper-bound grid.
@@ -135,11 +142,18 @@ struct GemmCfg {
 // registers (v_cvt_scalef32_pk_bf16_fp4: two values and their scale per
 // instruction, exact); everything else is the bf16 kernel, which then takes in
 // 4.25 KB instead of 16 KB of weights per CU and step.
-template <int RBT, typename C, bool GATE_UP, bool FP4>
+//
+// RS (row split) > 1 serves the last column tile of a matrix whose width is not
+// a multiple of the tile's: only NW / RS waves would have columns there, so the
+// waves form RS groups that share those columns and split the row blocks
+// (group rg takes row blocks rg, rg + RS, ...).  RBT is then the row blocks per
+// wave, RBT * RS are staged per step (blocks past the tile's rbt repeat its
+// last one and are not stored).
+template <int RBT, int RS, typename C, bool GATE_UP, bool FP4>
 __device__ __forceinline__ void gemm_tile(const uint4 *__restrict__ a_frag,  // [rb][KB][64]
                                           const uint4 *__restrict__ b_frag,  // expert: [nb][KB][64], FP4: [nb/2][KB/2][64]
                                           const uint16_t *__restrict__ b_scale,  // FP4: expert's [nb/2][KB/2][32] byte pairs
-                                          int KB, int rb0, int nb0, int nb_valid,
+                                          int KB, int rb0, int rbt, int nb0, int nb_valid,
                                           const float *__restrict__ bias_a,  // gate / down bias (expert)
                                           const float *__restrict__ bias_b,  // up bias (expert)
                                           void *__restrict__ outp, int out_ld, float limit,
@@ -161,7 +175,7 @@ __device__ __forceinline__ void gemm_tile(const uint4 *__restrict__ a_frag,  // 
   ring.p[4] = s4; ring.p[5] = s5; ring.p[6] = s6;
   constexpr int NBW = C::NBW, KPS = C::KPS, R = C::R, NW = C::NW;
   static_assert(KPS == 2, "the step is software-pipelined as two k blocks");
-  constexpr int A_CH = RBT * KPS;            // 1 KB chunks of the row operand per step
+  constexpr int A_CH = RBT * RS * KPS;       // 1 KB chunks of the row operand per step
   constexpr int LA = (A_CH + NW - 1) / NW;   // DMA loads per wave per step (a short last pass repeats a chunk)
   constexpr int LB = FP4 ? 2 : NBW * KPS;    // register loads per wave per step
   constexpr int LPS = LA + LB;
@@ -174,6 +188,9 @@ __device__ __forceinline__ void gemm_tile(const uint4 *__restrict__ a_frag,  // 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+  static_assert(NW % RS == 0 && RBT * RS <= C::RBT_MAX, "row split");
+  const int cw = RS == 1 ? w : w % (NW / RS);  // the wave's place among the columns
+  const int rg = RS == 1 ? 0 : w / (NW / RS);  // ... and among the row groups
 
   // The accumulators start from the bias (the up half of gate_up from bias + 1,
   // see swiglu_shifted).  gate_up computes the transposed product (weights as
@@ -189,7 +206,7 @@ __device__ __forceinline__ void gemm_tile(const uint4 *__restrict__ a_frag,  // 
     // a wave past the matrix's last column (last column tile only) reads the
     // last valid pair's bias: the expert's bias vector ends there
     const int P_last = ((nb0 + nb_valid) >> 1) - 1;
-    const int P0 = (nb0 + w * NBW) >> 1;
+    const int P0 = (nb0 + cw * NBW) >> 1;
 #pragma unroll
     for (int p = 0; p < NBW / 2; p++) {
       const int P = min(P0 + p, P_last);
@@ -203,7 +220,7 @@ __device__ __forceinline__ void gemm_tile(const uint4 *__restrict__ a_frag,  // 
   } else {
 #pragma unroll
     for (int j = 0; j < NBW; j++)
-      bias_d[j] = bias_a[kRowBlock * (nb0 + min(w * NBW + j, nb_valid - 1)) + (lane & 31)];
+      bias_d[j] = bias_a[kRowBlock * (nb0 + min(cw * NBW + j, nb_valid - 1)) + (lane & 31)];
   }
   f32x16 acc[RBT][NBW];
 
@@ -214,19 +231,20 @@ __device__ __forceinline__ void gemm_tile(const uint4 *__restrict__ a_frag,  // 
   const uint4 *b_src[NBW];
   const uint16_t *s_src = nullptr;
   if (FP4) {
-    const size_t pair = (size_t)((nb0 + min(w * NBW, nb_valid - NBW)) >> 1);
+    const size_t pair = (size_t)((nb0 + min(cw * NBW, nb_valid - NBW)) >> 1);
     b_src[0] = b_frag + pair * n_steps * 64 + lane;
     s_src = b_scale + pair * n_steps * 32 + (lane & 31);
   } else {
 #pragma unroll
     for (int j = 0; j < NBW; j++)
-      b_src[j] = b_frag + (size_t)(nb0 + min(w * NBW + j, nb_valid - 1)) * KB * 64 + lane;
+      b_src[j] = b_frag + (size_t)(nb0 + min(cw * NBW + j, nb_valid - 1)) * KB * 64 + lane;
   }
 
   // Row operand: chunk c of a step (c = pass*NW + wave) is row block c / KPS, k block c % KPS.
   auto issue_a = [&](uint4 *st, int ks, int m) {
     const int c = min(m * NW + w, A_CH - 1);
-    dma_to_lds_16(a_src + ((size_t)(c / KPS) * KB + ks * KPS + c % KPS) * 64, st + c * 64);
+    const int blk = RS == 1 ? c / KPS : min(c / KPS, rbt - 1);
+    dma_to_lds_16(a_src + ((size_t)blk * KB + ks * KPS + c % KPS) * 64, st + c * 64);
   };
   // Column operand: register m of a slot is column block m / KPS, k block m % KPS.
   // FP4: load 0 of a slot is the chunk of nibbles, load 1 the two scale bytes.
@@ -260,7 +278,7 @@ __device__ __forceinline__ void gemm_tile(const uint4 *__restrict__ a_frag,  // 
   // fragments of the next are read from LDS.
   bf16x8 fa[2][RBT];
   auto read_a = [&](const uint4 *st, int kk, int buf, int i) {
-    fa[buf][i] = __builtin_bit_cast(bf16x8, st[(i * KPS + kk) * 64 + lane]);
+    fa[buf][i] = __builtin_bit_cast(bf16x8, st[((i * RS + rg) * KPS + kk) * 64 + lane]);
   };
   auto mma = [](bf16x8 rows, bf16x8 colv, f32x16 c) {
     return GATE_UP ? __builtin_amdgcn_mfma_f32_32x32x16_bf16(colv, rows, c, 0, 0, 0)
@@ -411,7 +429,7 @@ __device__ __forceinline__ void gemm_tile(const uint4 *__restrict__ a_frag,  // 
 #undef MOE_WAIT_STEPS
 
   // Epilogue.
-  if (w * NBW >= nb_valid) return;  // a wave without columns (last column tile only)
+  if (cw * NBW >= nb_valid) return;  // a wave without columns (last column tile only)
   if (GATE_UP) {
     // Column blocks come in (gate, up) pairs (see pack_weight_kernel): blocks 2P
     // and 2P+1 of the product hold gate_j and up_j of j = 32P .. 32P+31 in the
@@ -424,10 +442,12 @@ __device__ __forceinline__ void gemm_tile(const uint4 *__restrict__ a_frag,  // 
     // fragment lane; nothing goes through LDS.
     uint4 *act = reinterpret_cast<uint4 *>(outp);
     const int kb2_total = out_ld / kFragK;
-    const int P0 = (nb0 + w * NBW) >> 1;                // first pair of this wave
-    const int pairs_valid = (nb_valid - w * NBW) >> 1;  // >= 1 here
+    const int P0 = (nb0 + cw * NBW) >> 1;                // first pair of this wave
+    const int pairs_valid = (nb_valid - cw * NBW) >> 1;  // >= 1 here
 #pragma unroll
     for (int i = 0; i < RBT; i++) {
+      const int blk = i * RS + rg;
+      if (RS > 1 && blk >= rbt) break;
 #pragma unroll
       for (int p = 0; p < NBW / 2; p++) {
         uint32_t pk[4][2];
@@ -439,7 +459,7 @@ __device__ __forceinline__ void gemm_tile(const uint4 *__restrict__ a_frag,  // 
                 swiglu_shifted(acc[i][2 * p][4 * g + 2 * d], acc[i][2 * p + 1][4 * g + 2 * d], limit),
                 swiglu_shifted(acc[i][2 * p][4 * g + 2 * d + 1], acc[i][2 * p + 1][4 * g + 2 * d + 1],
                                limit));
-        uint4 *dst = act + ((size_t)(rb0 + i) * kb2_total + 2 * (P0 + p)) * 64 + lane;
+        uint4 *dst = act + ((size_t)(rb0 + blk) * kb2_total + 2 * (P0 + p)) * 64 + lane;
 #pragma unroll
         for (int kb = 0; kb < 2; kb++) {
           // upper lane half of registers 8kb .. 8kb+3 <-> lower lane half of 8kb+4 .. 8kb+7
@@ -455,9 +475,11 @@ __device__ __forceinline__ void gemm_tile(const uint4 *__restrict__ a_frag,  // 
     float *ef = reinterpret_cast<float *>(epi + w * C::EPI_WAVE);
     const int n = lane & 31;
     const int rsub = 4 * (lane >> 5);
-    const int col0 = kRowBlock * (nb0 + w * NBW);
+    const int col0 = kRowBlock * (nb0 + cw * NBW);
 #pragma unroll
     for (int i = 0; i < RBT; i++) {
+      const int blk = i * RS + rg;
+      if (RS > 1 && blk >= rbt) break;
 #pragma unroll
       for (int j = 0; j < NBW; j++)
 #pragma unroll
@@ -465,14 +487,14 @@ __device__ __forceinline__ void gemm_tile(const uint4 *__restrict__ a_frag,  // 
           const int r = 8 * (q >> 2) + rsub + (q & 3);
           ef[r * LD + 32 * j + n] = acc[i][j][q];
         }
-      const size_t row0 = (size_t)(rb0 + i) * kRowBlock;
+      const size_t row0 = (size_t)(rb0 + blk) * kRowBlock;
 #pragma unroll
       for (int t = 0; t < NBW * 4; t++) {
         const int idx = t * 64 + lane;
         const int r = idx / (NBW * 8);
         const int c4 = idx % (NBW * 8);
         const float4 v = *reinterpret_cast<const float4 *>(ef + r * LD + 4 * c4);
-        if (w * NBW + c4 / 8 < nb_valid)
+        if (cw * NBW + c4 / 8 < nb_valid)
           *reinterpret_cast<float4 *>(y + (row0 + r) * out_ld + col0 + 4 * c4) = v;
       }
     }
@@ -503,9 +525,25 @@ __global__ __launch_bounds__(C::THREADS, C::WAVES) void grouped_gemm_kernel(
   const uint16_t *b_scale = FP4 ? w_scale + (size_t)tc.e * nb_total * KB * 8 : nullptr;
   const float *ba = bias_a + (size_t)tc.e * N;
   const float *bb = GATE_UP ? bias_b + (size_t)tc.e * N : nullptr;
-#define MOE_TILE(n) \
-  gemm_tile<n, C, GATE_UP, FP4>(a_frag, b_frag, b_scale, KB, tc.rb0, nb0, nb_valid, ba, bb, outp, N, limit, st0, st1, st2, st3, st4, st5, st6, epi)
+#define MOE_TILE_RS(n, rs) \
+  gemm_tile<n, rs, C, GATE_UP, FP4>(a_frag, b_frag, b_scale, KB, tc.rb0, tc.rbt, nb0, nb_valid, ba, bb, outp, N, limit, st0, st1, st2, st3, st4, st5, st6, epi)
+#define MOE_TILE(n) MOE_TILE_RS(n, 1)
   if constexpr (C::RBT_MAX == 8) {
+    // the last column tile, when only a quarter or half of the waves have columns in it
+    const int rs = row_split_of(nb_valid, C::NW, C::NBW);
+    if (!GATE_UP && rs == 4) {  // gate_up comes in (gate, up) pairs of pairs: never a quarter
+      if (tc.rbt <= 4) MOE_TILE_RS(1, 4); else MOE_TILE_RS(2, 4);
+      return;
+    }
+    if (rs == 2) {
+      switch ((tc.rbt + 1) >> 1) {
+        case 1: MOE_TILE_RS(1, 2); break;
+        case 2: MOE_TILE_RS(2, 2); break;
+        case 3: MOE_TILE_RS(3, 2); break;
+        default: MOE_TILE_RS(4, 2); break;
+      }
+      return;
+    }
     switch (tc.rbt) {
       case 1: MOE_TILE(1); break;
       case 2: MOE_TILE(2); break;
@@ -521,6 +559,7 @@ __global__ __launch_bounds__(C::THREADS, C::WAVES) void grouped_gemm_kernel(
     if (tc.rbt == 1) MOE_TILE(1); else MOE_TILE(2);
   }
 #undef MOE_TILE
+#undef MOE_TILE_RS
 }
 
 // 4 waves, one per SIMD, each 256 rows x 64 columns (8 x 2 accumulators = all
