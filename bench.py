@@ -78,10 +78,15 @@ def run_leg(shape, steps, warmup, device_timed=False):
     for _ in range(warmup):
         moe.forward(0, dx, None, T, dout)
     abi.sync()
-    moe.profile_enable(min(steps, 256))  # HIP events at the stage boundaries of the timed steps
+    # HIP events at the stage boundaries of the last few timed steps: an event
+    # between two kernels costs a few microseconds, so most steps run without.
+    n_prof = min(steps, 16)
+    moe.profile_enable(0)  # creates the events outside the timed region
     abi.sync()
     t0 = time.perf_counter()
-    for _ in range(steps):
+    for i in range(steps):
+        if i == steps - n_prof:
+            moe.profile_enable(n_prof)
         moe.forward(0, dx, None, T, dout)
     abi.sync()
     elapsed = time.perf_counter() - t0
@@ -100,8 +105,8 @@ def mxfp4_weight_bytes(shape):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--steps", type=int, default=500)
+    ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--workload", default="c2", help="c2 (headline), c3a, c3b, c4, c5 (MXFP4 decode)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-decode", action="store_true",
