@@ -292,28 +292,18 @@ __device__ __forceinline__ void gemm_tile(const uint4 *__restrict__ a_frag,  // 
       return __builtin_bit_cast(bf16x8, bq[slot][j * KPS + kk]);
     }
   };
-  // "all but the newest k steps have landed", k = 0 .. R-2
-#define MOE_WAIT_STEPS(k)                            \
-  switch (k) {                                       \
-    case 0: WAIT_VMCNT(0); break;                    \
-    case 1: WAIT_VMCNT(LPS * (R > 2 ? 1 : 0)); break; \
-    case 2: WAIT_VMCNT(LPS * (R > 3 ? 2 : 0)); break; \
-    case 3: WAIT_VMCNT(LPS * (R > 4 ? 3 : 0)); break; \
-    case 4: WAIT_VMCNT(LPS * (R > 5 ? 4 : 0)); break; \
-    default: WAIT_VMCNT(LPS * (R > 6 ? 5 : 0)); break; \
-  }
   static_assert(R == 7, "the step sequence below is written out for 7 slots");
 
   // Issue order per wave: A(0) B(0) A(1) B(1) ... ; at the top of step ks the row
-  // operand is issued through step ks+R-1 and the column operand through ks+R-2.
+  // operand is issued through step ks+R-1 and the column operand through ks+R-2
+  // (step indices past the tile's last are clamped to it).
+  const int last = n_steps - 1;
 #pragma unroll
   for (int s = 0; s < R - 1; s++) {
-    if (s < n_steps) {
 #pragma unroll
-      for (int m = 0; m < LA; m++) issue_a(ring.p[s], s, m);
+    for (int m = 0; m < LA; m++) issue_a(ring.p[s], min(s, last), m);
 #pragma unroll
-      for (int m = 0; m < LB; m++) issue_b(s, s, m);
-    }
+    for (int m = 0; m < LB; m++) issue_b(s, min(s, last), m);
   }
   if (GATE_UP) {
 #pragma unroll
@@ -336,13 +326,9 @@ __device__ __forceinline__ void gemm_tile(const uint4 *__restrict__ a_frag,  // 
 #pragma unroll
         for (int q = 0; q < 16; q++) acc[i][j][q] = bias_d[j];
   }
-  if (R - 1 < n_steps) {
 #pragma unroll
-    for (int m = 0; m < LA; m++) issue_a(ring.p[R - 1], R - 1, m);
-    WAIT_VMCNT(LPS * (R - 2) + LA);
-  } else {
-    WAIT_VMCNT(0);
-  }
+  for (int m = 0; m < LA; m++) issue_a(ring.p[R - 1], min(R - 1, last), m);
+  WAIT_VMCNT(LPS * (R - 2) + LA);
   lds_barrier();
 #pragma unroll
   for (int i = 0; i < RBT; i++) read_a(ring.p[0], 0, 0, i);
@@ -356,14 +342,18 @@ __device__ __forceinline__ void gemm_tile(const uint4 *__restrict__ a_frag,  // 
   //   wait until step ks+1 has arrived, barrier
   //   [MFMAs of k block 1 | DMA A(ks+R) into stage u, read row fragments of step ks+1]
   // The side work is spread over the MFMAs so that it issues in their shadow.
-  // STEADY steps (every refill exists) carry no branch at all, so the whole
-  // group of R steps is one straight block; the last steps of the tile run the
-  // same code with the refills guarded.
-  auto step = [&](auto u_c, auto steady_c, int ks) {
+  // Every step is the same straight code with the same count in its wait: the
+  // refills of the tile's last R-1 steps, for which there is nothing left to
+  // load, load its last step again (cache hits that nobody reads) instead of
+  // being skipped.  Skipping them costs more: with refills guarded at run time
+  // the waits can no longer be counted and the last six steps took twice their
+  // time (-3.4 % on gate_up, -4.9 % on down with the loads kept).  The wave
+  // ends with those loads in flight; s_endpgm waits for them.
+  auto step = [&](auto u_c, int ks) {
     constexpr int u = decltype(u_c)::value;
-    constexpr bool STEADY = decltype(steady_c)::value;
     const uint4 *cur = ring.p[u];
-    const bool refill_b = STEADY || ks + R - 1 < n_steps;
+    const int ks_b = min(ks + R - 1, last);
+    const int ks_a = min(ks + R, last);
 #pragma unroll
     for (int m = 0; m < NM; m++) {
 #pragma unroll
@@ -371,7 +361,7 @@ __device__ __forceinline__ void gemm_tile(const uint4 *__restrict__ a_frag,  // 
         if (t < RBT) {
           read_a(cur, 1, 1, t);
         } else if (t < RBT + LB) {
-          if (refill_b) issue_b((u + R - 1) % R, ks + R - 1, t - RBT);
+          issue_b((u + R - 1) % R, ks_b, t - RBT);
         } else if (t < RBT + LB + DEC) {
           decode(u, t - RBT - LB, 1);
         }
@@ -379,28 +369,19 @@ __device__ __forceinline__ void gemm_tile(const uint4 *__restrict__ a_frag,  // 
       acc[m / NBW][m % NBW] = mma(fa[0][m / NBW], cols_of(u, m % NBW, 0), acc[m / NBW][m % NBW]);
       __builtin_amdgcn_sched_barrier(0);
     }
-    const bool more = STEADY || ks + 1 < n_steps;
-    if (more) {
-      // loads issued after B(ks+1): steps ks+2 .. min(ks+R-1, n_steps-1)
-      if (STEADY) {
-        WAIT_VMCNT(LPS * (R - 2));
-      } else {
-        MOE_WAIT_STEPS(min(R - 2, n_steps - 2 - ks))
-      }
-      lds_barrier();  // step ks+1 is complete in LDS; every wave is done with stage u
-    }
-    const bool refill_a = STEADY || ks + R < n_steps;
+    WAIT_VMCNT(LPS * (R - 2));
+    lds_barrier();  // step ks+1 is complete in LDS; every wave is done with stage u
     const uint4 *nxt = ring.p[(u + 1) % R];
 #pragma unroll
     for (int m = 0; m < NM; m++) {
 #pragma unroll
       for (int t = m * SIDE2; t < (m + 1) * SIDE2; t++) {
         if (t < LA) {
-          if (refill_a) issue_a(ring.p[u], ks + R, t);
+          issue_a(ring.p[u], ks_a, t);
         } else if (t < LA + RBT) {
-          if (more) read_a(nxt, 0, 0, t - LA);
+          read_a(nxt, 0, 0, t - LA);
         } else if (t < LA + RBT + DEC) {
-          if (more) decode((u + 1) % R, t - LA - RBT, 0);  // landed: the wait above covers it
+          decode((u + 1) % R, t - LA - RBT, 0);  // landed: the wait above covers it
         }
       }
       acc[m / NBW][m % NBW] = mma(fa[1][m / NBW], cols_of(u, m % NBW, 1), acc[m / NBW][m % NBW]);
@@ -408,25 +389,21 @@ __device__ __forceinline__ void gemm_tile(const uint4 *__restrict__ a_frag,  // 
     }
   };
   int ks0 = 0;
-  for (; ks0 + 2 * R - 2 < n_steps; ks0 += R) {
-    step(IC<0>{}, std::true_type{}, ks0 + 0);
-    step(IC<1>{}, std::true_type{}, ks0 + 1);
-    step(IC<2>{}, std::true_type{}, ks0 + 2);
-    step(IC<3>{}, std::true_type{}, ks0 + 3);
-    step(IC<4>{}, std::true_type{}, ks0 + 4);
-    step(IC<5>{}, std::true_type{}, ks0 + 5);
-    step(IC<6>{}, std::true_type{}, ks0 + 6);
+  for (; ks0 + R <= n_steps; ks0 += R) {
+    step(IC<0>{}, ks0 + 0);
+    step(IC<1>{}, ks0 + 1);
+    step(IC<2>{}, ks0 + 2);
+    step(IC<3>{}, ks0 + 3);
+    step(IC<4>{}, ks0 + 4);
+    step(IC<5>{}, ks0 + 5);
+    step(IC<6>{}, ks0 + 6);
   }
-  for (; ks0 < n_steps; ks0 += R) {
-    if (ks0 + 0 < n_steps) step(IC<0>{}, std::false_type{}, ks0 + 0);
-    if (ks0 + 1 < n_steps) step(IC<1>{}, std::false_type{}, ks0 + 1);
-    if (ks0 + 2 < n_steps) step(IC<2>{}, std::false_type{}, ks0 + 2);
-    if (ks0 + 3 < n_steps) step(IC<3>{}, std::false_type{}, ks0 + 3);
-    if (ks0 + 4 < n_steps) step(IC<4>{}, std::false_type{}, ks0 + 4);
-    if (ks0 + 5 < n_steps) step(IC<5>{}, std::false_type{}, ks0 + 5);
-    if (ks0 + 6 < n_steps) step(IC<6>{}, std::false_type{}, ks0 + 6);
-  }
-#undef MOE_WAIT_STEPS
+  if (ks0 + 0 < n_steps) step(IC<0>{}, ks0 + 0);
+  if (ks0 + 1 < n_steps) step(IC<1>{}, ks0 + 1);
+  if (ks0 + 2 < n_steps) step(IC<2>{}, ks0 + 2);
+  if (ks0 + 3 < n_steps) step(IC<3>{}, ks0 + 3);
+  if (ks0 + 4 < n_steps) step(IC<4>{}, ks0 + 4);
+  if (ks0 + 5 < n_steps) step(IC<5>{}, ks0 + 5);
 
   // Epilogue.
   if (cw * NBW >= nb_valid) return;  // a wave without columns (last column tile only)
