@@ -315,7 +315,7 @@ __global__ __launch_bounds__(kDispThreads) void dispatch_scatter_kernel(
 // the rounds of 256 tokens play the part of the workgroups of the three-kernel
 // form (round r's assignments come after those of the rounds before it), so
 // the result is the same, bit for bit.
-constexpr int kSmallRounds = 2;
+constexpr int kSmallRounds = 1;
 
 __global__ __launch_bounds__(kDispThreads) void dispatch_small_kernel(
     const int *__restrict__ topk_i, const int *__restrict__ pos, int T, int E, int n_ct_gate_up,

@@ -149,11 +149,22 @@ struct GemmCfg {
 // (group rg takes row blocks rg, rg + RS, ...).  RBT is then the row blocks per
 // wave, RBT * RS are staged per step (blocks past the tile's rbt repeat its
 // last one and are not stored).
-template <int RBT, int RS, typename C, bool GATE_UP, bool FP4>
-__device__ __forceinline__ void gemm_tile(const uint4 *__restrict__ a_frag,  // [rb][KB][64]
+//
+// GATHER (gate_up of the small-batch configuration): there is no gathered copy
+// of the routed rows; the row operand's DMA reads the token rows themselves,
+// every lane at the address of its own row (rowmap) -- 32 bytes per row and
+// instruction instead of 1 KB in one piece.  That costs the main loop of a
+// large batch more than the gather kernel it saves (+25 % at 4096 tokens), but
+// when the GEMM is a stream of weights it is free and saves a launch and the
+// copy (-7 % per layer call at 64 tokens).  Such a DMA can complete after
+// register loads issued behind it, so here the waits count DMA only (see
+// WAIT_DMA_*).
+template <int RBT, int RS, typename C, bool GATE_UP, bool FP4, bool GATHER>
+__device__ __forceinline__ void gemm_tile(const uint4 *__restrict__ a_frag,  // [rb][KB][64]; GATHER: token rows [T][KB*2]
                                           const uint4 *__restrict__ b_frag,  // expert: [nb][KB][64], FP4: [nb/2][KB/2][64]
                                           const uint16_t *__restrict__ b_scale,  // FP4: expert's [nb/2][KB/2][32] byte pairs
                                           int KB, int rb0, int rbt, int nb0, int nb_valid,
+                                          const int *__restrict__ rowmap,    // GATHER: padded row -> assignment
                                           const float *__restrict__ bias_a,  // gate / down bias (expert)
                                           const float *__restrict__ bias_b,  // up bias (expert)
                                           void *__restrict__ outp, int out_ld, float limit,
@@ -226,6 +237,20 @@ __device__ __forceinline__ void gemm_tile(const uint4 *__restrict__ a_frag,  // 
 
   const int n_steps = KB / KPS;
   const uint4 *a_src = a_frag + (size_t)rb0 * KB * 64 + lane;
+  // GATHER: per DMA of a step, this lane's place in its token's row (16-byte
+  // units: a row is KB * 2 of them, a k block 2, the lane's half of it 1).
+  // Padding rows read token 0; their products are never used.
+  uint32_t lane_off[LA];
+  if (GATHER) {
+#pragma unroll
+    for (int m = 0; m < LA; m++) {
+      const int c = min(m * NW + w, A_CH - 1);
+      const int blk = RS == 1 ? c / KPS : min(c / KPS, rbt - 1);
+      const int a = rowmap[(rb0 + blk) * kRowBlock + (lane & 31)];
+      const int tok = a >= 0 ? a / kTopK : 0;
+      lane_off[m] = (uint32_t)tok * (uint32_t)(KB * 2) + (c % KPS) * 2 + (lane >> 5);
+    }
+  }
   // Column blocks past the end of the matrix (last column tile only) re-load
   // the last valid block; their products are never stored.
   const uint4 *b_src[NBW];
@@ -244,7 +269,11 @@ __device__ __forceinline__ void gemm_tile(const uint4 *__restrict__ a_frag,  // 
   auto issue_a = [&](uint4 *st, int ks, int m) {
     const int c = min(m * NW + w, A_CH - 1);
     const int blk = RS == 1 ? c / KPS : min(c / KPS, rbt - 1);
-    dma_to_lds_16(a_src + ((size_t)blk * KB + ks * KPS + c % KPS) * 64, st + c * 64);
+    if (GATHER) {
+      dma_to_lds_16(a_frag + lane_off[m] + ks * (KPS * 2), st + c * 64);
+    } else {
+      dma_to_lds_16(a_src + ((size_t)blk * KB + ks * KPS + c % KPS) * 64, st + c * 64);
+    }
   };
   // Column operand: register m of a slot is column block m / KPS, k block m % KPS.
   // FP4: load 0 of a slot is the chunk of nibbles, load 1 the two scale bytes.
@@ -293,6 +322,17 @@ __device__ __forceinline__ void gemm_tile(const uint4 *__restrict__ a_frag,  // 
     }
   };
   static_assert(R == 7, "the step sequence below is written out for 7 slots");
+  // "Step s of the row operand has landed" as a bound on the vector-memory
+  // counter.  The loads are issued in the order A(0) B(0) A(1) B(1) ... and
+  // complete in that order, so all but the newest n outstanding means step s has
+  // landed with n = everything issued behind it.  A scattered DMA (GATHER) was
+  // seen to complete after register loads issued behind it (whole tiles of
+  // wrong rows, run to run); there the bound counts the DMAs behind step s
+  // only, which holds whatever the register loads do and waits for some of them
+  // needlessly (free while the tile is a stream of weights, +30 % on tiles of
+  // 4 to 8 row blocks, which is why GATHER stays with the small batches).
+  constexpr int WAIT_DMA_FILL = GATHER ? LA * (R - 1) : LPS * (R - 2) + LA;  // A(0), A(0..R-1) issued
+  constexpr int WAIT_DMA_STEP = GATHER ? LA * (R - 2) : LPS * (R - 2);       // A(ks+1) at step ks
 
   // Issue order per wave: A(0) B(0) A(1) B(1) ... ; at the top of step ks the row
   // operand is issued through step ks+R-1 and the column operand through ks+R-2
@@ -304,6 +344,7 @@ __device__ __forceinline__ void gemm_tile(const uint4 *__restrict__ a_frag,  // 
     for (int m = 0; m < LA; m++) issue_a(ring.p[s], min(s, last), m);
 #pragma unroll
     for (int m = 0; m < LB; m++) issue_b(s, min(s, last), m);
+    __builtin_amdgcn_sched_barrier(0);  // the counted waits rely on this issue order
   }
   if (GATE_UP) {
 #pragma unroll
@@ -328,7 +369,7 @@ __device__ __forceinline__ void gemm_tile(const uint4 *__restrict__ a_frag,  // 
   }
 #pragma unroll
   for (int m = 0; m < LA; m++) issue_a(ring.p[R - 1], min(R - 1, last), m);
-  WAIT_VMCNT(LPS * (R - 2) + LA);
+  WAIT_VMCNT(WAIT_DMA_FILL);
   lds_barrier();
 #pragma unroll
   for (int i = 0; i < RBT; i++) read_a(ring.p[0], 0, 0, i);
@@ -369,7 +410,7 @@ __device__ __forceinline__ void gemm_tile(const uint4 *__restrict__ a_frag,  // 
       acc[m / NBW][m % NBW] = mma(fa[0][m / NBW], cols_of(u, m % NBW, 0), acc[m / NBW][m % NBW]);
       __builtin_amdgcn_sched_barrier(0);
     }
-    WAIT_VMCNT(LPS * (R - 2));
+    WAIT_VMCNT(WAIT_DMA_STEP);
     lds_barrier();  // step ks+1 is complete in LDS; every wave is done with stage u
     const uint4 *nxt = ring.p[(u + 1) % R];
 #pragma unroll
@@ -478,13 +519,14 @@ __device__ __forceinline__ void gemm_tile(const uint4 *__restrict__ a_frag,  // 
   }
 }
 
-template <typename C, bool GATE_UP, bool FP4>
+template <typename C, bool GATE_UP, bool FP4, bool GATHER>
 __global__ __launch_bounds__(C::THREADS, C::WAVES) void grouped_gemm_kernel(
     const uint4 *__restrict__ a_frag, const uint4 *__restrict__ w_frag,
     const uint16_t *__restrict__ w_scale,
     const float *__restrict__ bias_a, const float *__restrict__ bias_b,
-    const TileDesc *__restrict__ tiles, const int *__restrict__ totals, void *__restrict__ outp,
-    int K, int N, float limit) {
+    const TileDesc *__restrict__ tiles, const int *__restrict__ totals,
+    const int *__restrict__ rowmap, void *__restrict__ outp, int K, int N, float limit) {
+  static_assert(!GATHER || GATE_UP, "only the first GEMM reads token rows");
   constexpr int R = C::R;
   static_assert(R == 7, "seven stage arrays are declared below");
   __shared__ uint4 st0[C::STAGE], st1[C::STAGE], st2[C::STAGE], st3[C::STAGE], st4[C::STAGE],
@@ -503,7 +545,7 @@ __global__ __launch_bounds__(C::THREADS, C::WAVES) void grouped_gemm_kernel(
   const float *ba = bias_a + (size_t)tc.e * N;
   const float *bb = GATE_UP ? bias_b + (size_t)tc.e * N : nullptr;
 #define MOE_TILE_RS(n, rs) \
-  gemm_tile<n, rs, C, GATE_UP, FP4>(a_frag, b_frag, b_scale, KB, tc.rb0, tc.rbt, nb0, nb_valid, ba, bb, outp, N, limit, st0, st1, st2, st3, st4, st5, st6, epi)
+  gemm_tile<n, rs, C, GATE_UP, FP4, GATHER>(a_frag, b_frag, b_scale, KB, tc.rb0, tc.rbt, nb0, nb_valid, rowmap, ba, bb, outp, N, limit, st0, st1, st2, st3, st4, st5, st6, epi)
 #define MOE_TILE(n) MOE_TILE_RS(n, 1)
   if constexpr (C::RBT_MAX == 8) {
     // the last column tile, when only a quarter or half of the waves have columns in it
@@ -554,7 +596,7 @@ constexpr int kSmallBatchTokens = CfgGemmSmall::RBT_MAX * kRowBlock;
 
 // w_scale == nullptr: w holds bf16 fragments; otherwise w holds MXFP4 chunks and
 // w_scale their scale bytes (pack_fp4_kernel).
-template <typename C, bool GATE_UP>
+template <typename C, bool GATE_UP, bool GATHER = false>
 static hipError_t launch_gemm(const uint4 *a, const uint4 *w, const uint16_t *w_scale, const float *ba,
                               const float *bb, const DispatchBuffers &d, void *out, int K, int N,
                               float limit, int mt_cap, hipStream_t s) {
@@ -563,24 +605,25 @@ static hipError_t launch_gemm(const uint4 *a, const uint4 *w, const uint16_t *w_
   const int grid = kXcds * xcd_tile_cap(mt_cap * n_ct);
   const TileDesc *tiles = GATE_UP ? d.tiles_gate_up : d.tiles_down;
   if (w_scale) {
-    grouped_gemm_kernel<C, GATE_UP, true><<<grid, C::THREADS, 0, s>>>(a, w, w_scale, ba, bb, tiles,
-                                                                     d.totals, out, K, N, limit);
+    grouped_gemm_kernel<C, GATE_UP, true, GATHER><<<grid, C::THREADS, 0, s>>>(
+        a, w, w_scale, ba, bb, tiles, d.totals, d.rowmap, out, K, N, limit);
   } else {
-    grouped_gemm_kernel<C, GATE_UP, false><<<grid, C::THREADS, 0, s>>>(a, w, nullptr, ba, bb, tiles,
-                                                                      d.totals, out, K, N, limit);
+    grouped_gemm_kernel<C, GATE_UP, false, GATHER><<<grid, C::THREADS, 0, s>>>(
+        a, w, nullptr, ba, bb, tiles, d.totals, d.rowmap, out, K, N, limit);
   }
   return hipGetLastError();
 }
 
-hipError_t launch_gate_up(const uint16_t *xg, const void *w1, const uint16_t *w1_scale,
-                          const float *b1g, const float *b1u, const DispatchBuffers &d, uint16_t *act,
-                          int H, int IM, float limit, int mt_cap, int max_rows, hipStream_t s) {
-  if (max_rows <= kSmallBatchTokens)
-    return launch_gemm<CfgGemmSmall, true>(reinterpret_cast<const uint4 *>(xg),
-                                           reinterpret_cast<const uint4 *>(w1), w1_scale, b1g, b1u, d,
-                                           act, H, IM, limit, mt_cap, s);
-  return launch_gemm<CfgGemm, true>(reinterpret_cast<const uint4 *>(xg),
-                                    reinterpret_cast<const uint4 *>(w1), w1_scale, b1g, b1u, d, act, H,
+hipError_t launch_gate_up(const uint16_t *xg, const uint16_t *x, const void *w1,
+                          const uint16_t *w1_scale, const float *b1g, const float *b1u,
+                          const DispatchBuffers &d, uint16_t *act, int H, int IM, float limit, int mt_cap,
+                          int max_rows, hipStream_t s) {
+  static_assert(kSmallBatchTokens == kSmallBatchRows, "gate_up_gathers() and the small-batch configuration");
+  const uint4 *w = reinterpret_cast<const uint4 *>(w1);
+  if (gate_up_gathers(max_rows))
+    return launch_gemm<CfgGemmSmall, true, true>(reinterpret_cast<const uint4 *>(x), w, w1_scale, b1g, b1u,
+                                                 d, act, H, IM, limit, mt_cap, s);
+  return launch_gemm<CfgGemm, true>(reinterpret_cast<const uint4 *>(xg), w, w1_scale, b1g, b1u, d, act, H,
                                     IM, limit, mt_cap, s);
 }
 

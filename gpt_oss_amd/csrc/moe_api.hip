@@ -138,9 +138,9 @@ int run_experts(moe_handle *h, int layer, const uint16_t *x, const int *pos, con
   HIP_TRY(tm.mark(MOE_STAGE_DISPATCH));
   HIP_TRY(launch_dispatch(topk_i, pos, T, c.experts, gate_up_col_tiles(c), down_col_tiles(c), h->disp, s));
   HIP_TRY(tm.mark(MOE_STAGE_GATHER));
-  HIP_TRY(launch_gather(x, h->disp, h->xg, T, c.hidden, rb_cap, s));
+  if (!gate_up_gathers(max_rows)) HIP_TRY(launch_gather(x, h->disp, h->xg, T, c.hidden, rb_cap, s));
   HIP_TRY(tm.mark(MOE_STAGE_GATE_UP));
-  HIP_TRY(launch_gate_up(h->xg, lw.w1q ? static_cast<const void *>(lw.w1q) : lw.w1, lw.w1s, lw.b1g,
+  HIP_TRY(launch_gate_up(h->xg, x, lw.w1q ? static_cast<const void *>(lw.w1q) : lw.w1, lw.w1s, lw.b1g,
                          lw.b1u, h->disp, h->act, c.hidden, c.inter, c.swiglu_limit, mt_cap, max_rows, s));
   HIP_TRY(tm.mark(MOE_STAGE_DOWN));
   HIP_TRY(launch_down(h->act, lw.w2q ? static_cast<const void *>(lw.w2q) : lw.w2, lw.w2s, lw.b2,

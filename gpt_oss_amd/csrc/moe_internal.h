@@ -114,9 +114,16 @@ hipError_t launch_gather(const uint16_t *x, const DispatchBuffers &d, uint16_t *
                          int rb_cap, hipStream_t s);
 
 // w*_scale == nullptr: w* are bf16 fragments; otherwise MXFP4 chunks + scale bytes.
-hipError_t launch_gate_up(const uint16_t *xg, const void *w1, const uint16_t *w1_scale,
-                          const float *b1g, const float *b1u, const DispatchBuffers &d, uint16_t *act,
-                          int H, int IM, float limit, int mt_cap, int max_rows, hipStream_t s);
+// When no expert can have more than this many rows (the small-batch
+// configuration of the GEMMs) the gate_up GEMM reads the token rows itself,
+// through rowmap, and launch_gather is not needed; above, it reads the gathered
+// copy xg.
+constexpr int kSmallBatchRows = 64;
+inline bool gate_up_gathers(int max_rows) { return max_rows <= kSmallBatchRows; }
+hipError_t launch_gate_up(const uint16_t *xg, const uint16_t *x, const void *w1,
+                          const uint16_t *w1_scale, const float *b1g, const float *b1u,
+                          const DispatchBuffers &d, uint16_t *act, int H, int IM, float limit, int mt_cap,
+                          int max_rows, hipStream_t s);
 hipError_t launch_down(const uint16_t *act, const void *w2, const uint16_t *w2_scale, const float *b2,
                        const DispatchBuffers &d, float *y, int H, int IM, int mt_cap, int max_rows,
                        hipStream_t s);

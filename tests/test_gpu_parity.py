@@ -318,6 +318,38 @@ def test_c5_mxfp4_ingest():
         m4.upload_layer_mxfp4(3, wr, br, b1k, s1, b1, b2k, s2, b2)  # layer out of range
 
 
+def test_small_batches_repeat_bit_for_bit():
+    """Batches of at most 64 tokens take paths of their own (one-workgroup
+    dispatch, gate_up reading the token rows through the row map, GEMMs built
+    for several workgroups per CU).  Twelve calls in a row must give the same
+    bits, with MXFP4 and with bf16 weights, and the two must agree (the MXFP4
+    values are exact in bf16): a row operand read before it had landed showed
+    as whole token rows that differed from run to run."""
+    sh = synth.CONFIGS["c5"]
+    wr, br = (synth.round_bf16(a) for a in synth.make_router(sh))
+    b1k, s1, b1, b2k, s2, b2 = synth.make_experts_mxfp4(sh)
+    w1, w2 = ob.mxfp4_dequant(b1k, s1), ob.mxfp4_dequant(b2k, s2)
+    m4 = abi.Moe(sh.hidden, sh.inter, sh.experts, max_tokens=sh.tokens, swiglu_limit=sh.limit)
+    m4.upload_layer_mxfp4(0, wr, br, b1k, s1, b1, b2k, s2, b2)
+    m16 = abi.Moe(sh.hidden, sh.inter, sh.experts, max_tokens=sh.tokens, swiglu_limit=sh.limit)
+    m16.upload_layer(0, wr, br, w1, b1, w2, b2)
+    for T in (sh.tokens, 16, 1):
+        x = synth.round_bf16(synth.make_activations(sh, seed=T, tokens=T))
+        dx = abi.DevBuf.from_numpy(synth.to_bf16_bits(x))
+        dout = abi.DevBuf(T * sh.hidden * 4)
+        first = None
+        for m in (m4, m16):
+            for _ in range(12):
+                dout.memset(0xFF)
+                m.forward(0, dx, None, T, dout)
+                abi.sync()
+                got = dout.download((T, sh.hidden), np.float32)
+                assert np.isfinite(got).all()
+                if first is None:
+                    first = got
+                assert np.array_equal(got, first), f"{T} tokens: a repeated call gave other bits"
+
+
 def test_ffn_block_in_place(c2):
     """moe_block_forward: RMS norm in front, residual add behind, in place on a
     bf16 stream.  The norm is checked through the routing it leads to (bit-exact
