@@ -27,11 +27,17 @@ sys.path.insert(0, ROOT)
 
 PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0
+# What the box itself reaches with no algorithm in the way (second denominators,
+# reported next to the published peaks): v_mfma_f32_32x32x16_bf16 from registers
+# on all 256 CUs (profiles/mfma_register_rate.md) and a plain read stream over
+# 2 GB (profiles/l2_ingest_ceiling.md).
+MEASURED_MFMA_TFLOPS = 1880.0
+MEASURED_HBM_STREAM_GBS = 6150.0
 
 # HBM bytes per gate_up launch at the c2 workload from rocprofv3 --pmc
 # (FETCH_SIZE + WRITE_SIZE, scaled by the same counters on a copy kernel);
 # None until measured for the workload being run.
-MEASURED_TRAFFIC_BYTES = {"c2": 1.552e9}  # profiles/bench_c2_counters.md
+MEASURED_TRAFFIC_BYTES = {"c2": 1.706e9, "c5": 0.290e9}  # profiles/bench_c2_counters.md, bench_c5_mxfp4_decode.md
 
 
 def cpu_baseline(shape, L, budget_s=15.0):
@@ -138,12 +144,16 @@ def main():
         achieved = mxfp4_weight_bytes(shape) * 2 / 3 / (stages["gate_up"] * 1e-3) / 1e9
         roofline = {"bound": "hbm", "kernel": "grouped_gemm_kernel<gate_up, MXFP4>",
                     "achieved": achieved, "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                    "frac": achieved / PEAK_HBM_GBS, "traffic": MEASURED_TRAFFIC_BYTES.get(shape.name)}
+                    "frac": achieved / PEAK_HBM_GBS, "traffic": MEASURED_TRAFFIC_BYTES.get(shape.name),
+                    "measured_peak": MEASURED_HBM_STREAM_GBS,
+                    "frac_of_measured_peak": achieved / MEASURED_HBM_STREAM_GBS}
     else:
         achieved = flops_gate_up / (stages["gate_up"] * 1e-3) / 1e12
         roofline = {"bound": "mfma", "kernel": "grouped_gemm_kernel<gate_up>",
                     "achieved": achieved, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                    "frac": achieved / PEAK_BF16_TFLOPS, "traffic": MEASURED_TRAFFIC_BYTES.get(shape.name)}
+                    "frac": achieved / PEAK_BF16_TFLOPS, "traffic": MEASURED_TRAFFIC_BYTES.get(shape.name),
+                    "measured_peak": MEASURED_MFMA_TFLOPS,
+                    "frac_of_measured_peak": achieved / MEASURED_MFMA_TFLOPS}
     weights = "MXFP4 expert weights" if mxfp4 else "bf16 weights"
     result = {
         "metric": "MoE-layer tokens/sec",
