@@ -22,9 +22,11 @@
 //     ring by DMA (global_load_lds_dwordx4), R-1 steps ahead of the MFMAs;
 //   * the column operand is private to a wave in this layout, so it never
 //     touches LDS: it is loaded into an R-slot ring of VGPRs, R-1 steps ahead.
-// With R = 7 that is 6 steps x 32 KB = 192 KB in flight per CU.  Loads return
-// in order, so waiting for "all but the newest n" (s_waitcnt vmcnt(n)) picks out
-// exactly the step that is needed next and leaves the later ones in flight.
+// With R = 7 that is 6 steps x 32 KB = 192 KB in flight per CU.  These loads
+// complete in the order they were issued, so waiting for "all but the newest n"
+// (s_waitcnt vmcnt(n)) picks out exactly the step that is needed next and
+// leaves the later ones in flight (the scattered DMA of the GATHER variant is
+// the exception, see there).
 // Measured in the steady loop: 1113 clocks per step of 1024 MFMA clocks (tile of
 // 8 row blocks), the same in every group of every tile.
 //
