@@ -37,7 +37,7 @@ MEASURED_HBM_STREAM_GBS = 6150.0
 # HBM bytes per gate_up launch at the c2 workload from rocprofv3 --pmc
 # (FETCH_SIZE + WRITE_SIZE, scaled by the same counters on a copy kernel);
 # None until measured for the workload being run.
-MEASURED_TRAFFIC_BYTES = {"c2": 1.706e9, "c5": 0.290e9}  # profiles/bench_c2_counters.md, bench_c5_mxfp4_decode.md
+MEASURED_TRAFFIC_BYTES = {"c2": 1.70e9, "c5": 0.290e9}  # profiles/bench_c2_counters.md, bench_c5_mxfp4_decode.md
 
 
 def cpu_baseline(shape, L, budget_s=15.0):
