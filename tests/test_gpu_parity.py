@@ -271,6 +271,27 @@ def test_all_tokens_on_four_experts_and_tiny_batches(c2):
         check_outputs(R, L2, x, None, np.arange(T))
 
 
+@pytest.mark.parametrize("T", [16, 17, 64, 65, 256, 257])
+def test_batch_size_boundaries(c2, T):
+    """Either side of the sizes at which the library changes its plan: up to 64
+    rows per expert the GEMMs run in their small-batch configuration and gate_up
+    reads the token rows itself, up to 256 tokens the dispatch is one workgroup.
+    moe_forward bounds the rows per expert by T, moe_experts (whose ids come from
+    the caller) by 4 T, so between 17 and 64 tokens the two entry points take
+    different configurations for the same work: same bits required."""
+    sh, L, m = c2
+    x = L["x"][500:500 + T]
+    R = abi.run_layer(m, 0, x, None)
+    check_routing(R, L, x, None, sh.experts)
+    check_outputs(R, L, x, None, np.arange(min(T, 24)))
+    dx = abi.DevBuf.from_numpy(synth.to_bf16_bits(x))
+    dti, dtv = abi.DevBuf.from_numpy(R["topk_i"]), abi.DevBuf.from_numpy(R["topk_v"])
+    dout = abi.DevBuf(T * sh.hidden * 4)
+    m.experts(0, dx, None, dti, dtv, T, dout, accumulate=False)
+    abi.sync()
+    assert np.array_equal(dout.download((T, sh.hidden), np.float32), R["out"])
+
+
 def test_c4_120b_shape():
     sh = synth.CONFIGS["c4"]
     L = bf16_layer(sh)
