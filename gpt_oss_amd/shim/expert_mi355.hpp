@@ -2,7 +2,8 @@
 // of libmi355_moe (include/moe_abi.h).  It is meant to be #included from the
 // reference's getp-csrc/getp_run.cpp (after common/defines.h, which provides
 // DeviceContext, Transformer, model_config and HIP_CHECK) in place of the MoE
-// kernels it launches; INTEGRATION.md shows the exact edits.
+// kernels it launches: one call in init_device_context, one in the layer loop
+// of gpu_forward_device_batch, one in cleanup_device_context.
 //
 // Mirrored interfaces (reference file:line):
 //   mi355_moe_init      <- expert upload of init_device_context (getp_run.cpp:186-293)
