@@ -11,16 +11,6 @@ namespace moe {
 
 constexpr int kDispThreads = 256;  // tokens per workgroup in count / scatter
 
-__device__ __forceinline__ uint16_t f32_to_bf16_rne_disp(float f) {
-  uint32_t u = __float_as_uint(f);
-  if (~u & 0x7f800000u) {
-    u += 0x7fffu + ((u >> 16) & 1u);
-  } else if (u & 0xffffu) {
-    u |= 0x10000u;
-  }
-  return (uint16_t)(u >> 16);
-}
-
 // Pass 1: per-workgroup histogram of expert ids over active rows.  Also resets
 // rowmap and perm to -1 (a fill kernel rather than a memset so that the call
 // sequence can be captured in a graph).
@@ -479,8 +469,8 @@ __global__ __launch_bounds__(256) void combine_kernel(const float *__restrict__ 
       const uint2 xv = xr[c];
       const float r0 = __uint_as_float(xv.x << 16) + s.x, r1 = __uint_as_float(xv.x & 0xffff0000u) + s.y;
       const float r2 = __uint_as_float(xv.y << 16) + s.z, r3 = __uint_as_float(xv.y & 0xffff0000u) + s.w;
-      xr[c] = make_uint2(f32_to_bf16_rne_disp(r0) | ((uint32_t)f32_to_bf16_rne_disp(r1) << 16),
-                         f32_to_bf16_rne_disp(r2) | ((uint32_t)f32_to_bf16_rne_disp(r3) << 16));
+      xr[c] = make_uint2(f32_to_bf16_rne(r0) | ((uint32_t)f32_to_bf16_rne(r1) << 16),
+                         f32_to_bf16_rne(r2) | ((uint32_t)f32_to_bf16_rne(r3) << 16));
     } else {
       o[c] = s;
     }

@@ -9,6 +9,18 @@
 
 namespace moe {
 
+// float -> bf16 bits, round to nearest even; a NaN stays a NaN
+// (/opt/rocm/include/hip/amd_detail/amd_hip_bfloat16.h:96-131).
+__device__ __forceinline__ uint16_t f32_to_bf16_rne(float f) {
+  uint32_t u = __float_as_uint(f);
+  if (~u & 0x7f800000u) {
+    u += 0x7fffu + ((u >> 16) & 1u);
+  } else if (u & 0xffffu) {
+    u |= 0x10000u;
+  }
+  return (uint16_t)(u >> 16);
+}
+
 constexpr int kTopK = 4;        // EXPERT_PER_TOKEN, common/defines.h:27
 constexpr int kRowBlock = 32;   // rows of one MFMA fragment (v_mfma_f32_32x32x16_bf16)
 constexpr int kFragK = 16;      // reduction depth of one fragment

@@ -11,16 +11,6 @@
 
 namespace moe {
 
-__device__ __forceinline__ uint16_t f32_to_bf16_rne_norm(float f) {
-  uint32_t u = __float_as_uint(f);
-  if (~u & 0x7f800000u) {
-    u += 0x7fffu + ((u >> 16) & 1u);
-  } else if (u & 0xffffu) {
-    u |= 0x10000u;
-  }
-  return (uint16_t)(u >> 16);
-}
-
 // One wave per token, 8 elements (16 bytes) per lane and pass.
 __global__ __launch_bounds__(256) void rmsnorm_kernel(const uint16_t *__restrict__ x,
                                                      const float *__restrict__ weight,
@@ -63,7 +53,7 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(const uint16_t *__restrict
       const float a = __uint_as_float(u[i] << 16), b = __uint_as_float(u[i] & 0xffff0000u);
       const float ra = (float)((double)w[2 * i] * ((double)scale * (double)a));
       const float rb = (float)((double)w[2 * i + 1] * ((double)scale * (double)b));
-      o[i] = f32_to_bf16_rne_norm(ra) | ((uint32_t)f32_to_bf16_rne_norm(rb) << 16);
+      o[i] = f32_to_bf16_rne(ra) | ((uint32_t)f32_to_bf16_rne(rb) << 16);
     }
     out[c] = make_uint4(o[0], o[1], o[2], o[3]);
   }

@@ -7,16 +7,6 @@
 
 namespace moe {
 
-__device__ __forceinline__ uint16_t f32_to_bf16_rne(float f) {
-  uint32_t u = __float_as_uint(f);
-  if (~u & 0x7f800000u) {
-    u += 0x7fffu + ((u >> 16) & 1u);
-  } else if (u & 0xffffu) {
-    u |= 0x10000u;
-  }
-  return (uint16_t)(u >> 16);
-}
-
 __device__ __forceinline__ float bf16_round(float f) {
   return __uint_as_float((uint32_t)f32_to_bf16_rne(f) << 16);
 }
