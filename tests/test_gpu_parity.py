@@ -371,13 +371,14 @@ def test_small_batches_repeat_bit_for_bit():
                 assert np.array_equal(got, first), f"{T} tokens: a repeated call gave other bits"
 
 
-def test_ffn_block_in_place(c2):
+@pytest.mark.parametrize("T", [1024, 48])
+def test_ffn_block_in_place(c2, T):
     """moe_block_forward: RMS norm in front, residual add behind, in place on a
     bf16 stream.  The norm is checked through the routing it leads to (bit-exact
     offsets and permutation need bit-exact normalised rows up to near-ties), the
-    result against the oracle's composition of the same steps."""
+    result against the oracle's composition of the same steps.  48 tokens take
+    the small-batch path, whose gate_up reads the normalised rows directly."""
     sh, L, m = c2
-    T = 1024
     rng = np.random.default_rng(21)
     x = synth.round_bf16((rng.standard_normal((T, sh.hidden)) * rng.uniform(0.5, 4.0, (T, 1))).astype(np.float32))
     rw = synth.round_bf16((1 + 0.1 * rng.standard_normal(sh.hidden)).astype(np.float32))
@@ -400,7 +401,7 @@ def test_ffn_block_in_place(c2):
     assert np.array_equal(off, off_o) and np.array_equal(perm[:off_o[-1]], perm_o)
 
     rows = np.sort(rng.choice(T, 24, replace=False))
-    want, _ = ob.ffn_block(x[rows], pos[rows], rw, *[L[k] for k in W], 4, sh.limit,
+    want, _ = ob.ffn_block(np.ascontiguousarray(x[rows]), np.ascontiguousarray(pos[rows]), rw, *[L[k] for k in W], 4, sh.limit,
                            mode=ob.ROUND_ACT_BF16 | ob.PAR_TOKENS)
     # one bf16 step of the result on top of the layer's bar
     tol = MAX_ABS + 2.0 ** -7 * np.abs(want)
