@@ -54,6 +54,8 @@ struct moe_handle {
   // routing produced by the router stage (or copied from the caller)
   int *topk_i = nullptr;
   float *topk_v = nullptr;
+  double *router_ws = nullptr;     // sums of the router's shared-tile form
+  int *router_arrivals = nullptr;  // its arrival counters, zero between launches
   // dispatch
   DispatchBuffers disp{};
   int a_cap = 0;      // max assignments
@@ -199,6 +201,8 @@ int moe_create(const moe_config *cfg, moe_handle **out) {
   if (rc == MOE_OK) rc = dev_alloc(h, &(ptr), (count), true)
   ALLOC(h->topk_i, (size_t)h->a_cap);
   ALLOC(h->topk_v, (size_t)h->a_cap);
+  ALLOC(h->router_ws, (size_t)kRouterSplitTiles * kRouterSplitMax * h->E_pad * 16);
+  ALLOC(h->router_arrivals, (size_t)kRouterSplitTiles);
   ALLOC(h->disp.blk_counts, (size_t)h->n_blk_cap * E);
   ALLOC(h->disp.offsets, (size_t)E + 1);
   ALLOC(h->disp.perm, (size_t)h->a_cap);
@@ -218,6 +222,10 @@ int moe_create(const moe_config *cfg, moe_handle **out) {
   ALLOC(h->y, (size_t)h->a_pad_cap * H);
 #undef ALLOC
   h->disp.a_pad_cap = h->a_pad_cap;
+  if (rc == MOE_OK) {
+    const hipError_t e0 = hipMemset(h->router_arrivals, 0, kRouterSplitTiles * sizeof(int));
+    if (e0 != hipSuccess) rc = fail(MOE_ERR_HIP, "hipMemset failed: %s", hipGetErrorString(e0));
+  }
   if (rc != MOE_OK) {
     moe_destroy(h);
     return rc;
@@ -237,6 +245,7 @@ int moe_destroy(moe_handle *h) {
     (void)hipFree(lw.w1q); (void)hipFree(lw.w1s); (void)hipFree(lw.w2q); (void)hipFree(lw.w2s);
   }
   (void)hipFree(h->topk_i); (void)hipFree(h->topk_v);
+  (void)hipFree(h->router_ws); (void)hipFree(h->router_arrivals);
   (void)hipFree(h->disp.blk_counts); (void)hipFree(h->disp.offsets); (void)hipFree(h->disp.perm);
   (void)hipFree(h->disp.rowmap); (void)hipFree(h->disp.inv); (void)hipFree(h->disp.info); (void)hipFree(h->disp.totals);
   (void)hipFree(h->disp.tiles_gate_up); (void)hipFree(h->disp.tiles_down);
@@ -398,7 +407,8 @@ int moe_router(moe_handle *h, int layer, const uint16_t *x, const int *pos, int 
   if (n_tokens == 0) return MOE_OK;
   const LayerWeights &lw = h->layers[layer];
   HIP_TRY(launch_router(x, pos, lw.wr, lw.br, n_tokens, h->cfg.hidden, h->cfg.experts, h->E_pad,
-                        score, topk_i, topk_v, static_cast<hipStream_t>(stream)));
+                        score, topk_i, topk_v, h->router_ws, h->router_arrivals,
+                        static_cast<hipStream_t>(stream)));
   return MOE_OK;
 }
 
@@ -452,7 +462,7 @@ int moe_forward(moe_handle *h, int layer, const uint16_t *x, const int *pos, int
   StageTimer tm(h, s);
   HIP_TRY(tm.mark(MOE_STAGE_ROUTER));
   HIP_TRY(launch_router(x, pos, lw.wr, lw.br, n_tokens, h->cfg.hidden, h->cfg.experts, h->E_pad,
-                        nullptr, h->topk_i, h->topk_v, s));
+                        nullptr, h->topk_i, h->topk_v, h->router_ws, h->router_arrivals, s));
   rc = run_experts(h, layer, x, pos, h->topk_i, h->topk_v, n_tokens, n_tokens, out, accumulate, s, tm);
   if (rc == MOE_OK) tm.done();
   return rc;
@@ -494,7 +504,7 @@ int moe_block_forward(moe_handle *h, int layer, uint16_t *x, const int *pos, int
   HIP_TRY(tm.mark(MOE_STAGE_ROUTER));  // the norm is counted with the router stage
   HIP_TRY(launch_rmsnorm(x, lw.rms_w, pos, h->t_norm, n_tokens, h->cfg.hidden, s));
   HIP_TRY(launch_router(h->t_norm, pos, lw.wr, lw.br, n_tokens, h->cfg.hidden, h->cfg.experts,
-                        h->E_pad, nullptr, h->topk_i, h->topk_v, s));
+                        h->E_pad, nullptr, h->topk_i, h->topk_v, h->router_ws, h->router_arrivals, s));
   rc = run_experts(h, layer, h->t_norm, pos, h->topk_i, h->topk_v, n_tokens, n_tokens, nullptr, 0, s, tm,
                    x);
   if (rc == MOE_OK) tm.done();

@@ -103,9 +103,15 @@ hipError_t launch_pack_fp4(const uint8_t *blocks, const uint8_t *scales, uint8_t
 hipError_t launch_pack_bias(const float *src, float *dst_a, float *dst_b, int n, bool deinterleave,
                             hipStream_t s);
 
-hipError_t launch_router(const uint16_t *x, const int *pos, const uint16_t *wr, const float *br,
-                         int T, int H, int E, int E_pad, float *score, int *topk_i, float *topk_v,
-                         hipStream_t s);
+// ws / arrivals: workspace of the router's shared-tile form (kRouterSplitTiles *
+// kRouterSplitMax * E_pad * 16 doubles; kRouterSplitTiles ints, zero before the
+// first launch and left zero by every launch); ws == nullptr keeps one
+// workgroup per 16 tokens.
+constexpr int kRouterSplitTiles = 8;   // batches of at most this many tiles of 16 tokens share tiles
+constexpr int kRouterSplitMax = 16;    // workgroups per shared tile, at most
+hipError_t launch_router(const uint16_t *x, const int *pos, const uint16_t *wr, const float *br, int T,
+                         int H, int E, int E_pad, float *score, int *topk_i, float *topk_v,
+                         double *ws, int *arrivals, hipStream_t s);
 
 struct DispatchBuffers {
   int *blk_counts;    // [n_blk, E]

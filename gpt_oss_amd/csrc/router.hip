@@ -32,14 +32,22 @@ __device__ __forceinline__ void widen8(const uint4 v, double (&d)[8]) {
 // dimension in chunks of 32 (wave w takes chunks w, w+WPC, ...), each wave
 // keeps NT 16x16 accumulators, and the partial sums are added in wave order
 // through LDS.  NT = E_pad / 16.
-template <int NT, int WPC, int D>
+//
+// SPLIT (small batches: a handful of workgroups would otherwise carry all the
+// fp64 MFMAs on as many CUs, 20 us whatever the batch): gridDim.y workgroups
+// share a tile of 16 tokens, each taking `cps` consecutive chunks.  They leave
+// their sums in `ws`; the one that arrives last (a counter per tile) adds them
+// up in the order of the chunks -- the same sum whichever arrives last -- and
+// selects.  No workgroup waits for another.
+template <int NT, int WPC, int D, bool SPLIT>
 __global__ __launch_bounds__(WPC * 64) void router_kernel(
     const uint16_t *__restrict__ x, const int *__restrict__ pos, const uint16_t *__restrict__ wr,
     const float *__restrict__ br, int T, int H, int E, float *__restrict__ score,
-    int *__restrict__ topk_i, float *__restrict__ topk_v) {
+    int *__restrict__ topk_i, float *__restrict__ topk_v, double *ws, int *arrivals, int cps) {
   constexpr int E_pad = NT * 16;
   __shared__ double part[WPC][NT][4][64];  // [wave][expert block][reg][lane]
   __shared__ float logits[16][E_pad + 1];
+  __shared__ int is_last;
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -49,6 +57,8 @@ __global__ __launch_bounds__(WPC * 64) void router_kernel(
   const int g = lane >> 4;    // which 8 of the chunk's 32 k this lane holds
   const int t_ld = min(tok0 + row, T - 1);
   const int kc_total = H / 32;
+  const int c_begin = SPLIT ? (int)blockIdx.y * cps : 0;
+  const int c_end = SPLIT ? min(c_begin + cps, kc_total) : kc_total;
 
   f64x4 acc[NT];
 #pragma unroll
@@ -60,21 +70,21 @@ __global__ __launch_bounds__(WPC * 64) void router_kernel(
   // round trips.  Past the end the ring re-loads the last chunk and drops it.
   const uint16_t *xrow = x + (size_t)t_ld * H + g * 8;
   const uint16_t *wlane = wr + (size_t)lane * 8;
-  uint4 xs[D], ws[D][NT];
+  uint4 xs[D], wq[D][NT];
   auto load = [&](int d, int c) {
-    const int cc = min(c, kc_total - 1);
+    const int cc = min(c, c_end - 1);
     xs[d] = *reinterpret_cast<const uint4 *>(xrow + cc * 32);
 #pragma unroll
     for (int n = 0; n < NT; n++)
-      ws[d][n] = *reinterpret_cast<const uint4 *>(wlane + ((size_t)n * kc_total + cc) * 512);
+      wq[d][n] = *reinterpret_cast<const uint4 *>(wlane + ((size_t)n * kc_total + cc) * 512);
   };
 #pragma unroll
-  for (int d = 0; d < D; d++) load(d, w + d * WPC);
-  for (int c0 = w; c0 < kc_total; c0 += D * WPC) {
+  for (int d = 0; d < D; d++) load(d, c_begin + w + d * WPC);
+  for (int c0 = c_begin + w; c0 < c_end; c0 += D * WPC) {
 #pragma unroll
     for (int d = 0; d < D; d++) {
       const int c = c0 + d * WPC;
-      if (c < kc_total) {  // the same for the whole wave
+      if (c < c_end) {  // the same for the whole wave
         double xd[8];
         widen8(xs[d], xd);
         // Two accumulators are advanced alternately so that back-to-back MFMAs do
@@ -84,7 +94,7 @@ __global__ __launch_bounds__(WPC * 64) void router_kernel(
         for (int n = 0; n < NT; n += NP) {
           double wd[NP][8];
 #pragma unroll
-          for (int p = 0; p < NP; p++) widen8(ws[d][n + p], wd[p]);
+          for (int p = 0; p < NP; p++) widen8(wq[d][n + p], wd[p]);
 #pragma unroll
           for (int s = 0; s < 8; s++)
 #pragma unroll
@@ -103,14 +113,42 @@ __global__ __launch_bounds__(WPC * 64) void router_kernel(
   }
   __syncthreads();
 
+  if (SPLIT) {
+    const int S = gridDim.y;
+    double *mine = ws + ((size_t)blockIdx.x * S + blockIdx.y) * (NT * 256);
+    for (int idx = tid; idx < NT * 4 * 64; idx += WPC * 64) {
+      double s = 0.0;
+#pragma unroll
+      for (int ww = 0; ww < WPC; ww++) s += (&part[ww][0][0][0])[idx];
+      mine[idx] = s;
+    }
+    __threadfence();  // the sums are out before the arrival is counted
+    __syncthreads();
+    if (tid == 0) is_last = atomicAdd(&arrivals[blockIdx.x], 1) == S - 1;
+    __syncthreads();
+    if (!is_last) return;
+    __threadfence();  // and the other workgroups' sums are read after it
+  }
+
   // Result register i of lane l is token 4*i + l/16, expert 16*n + l%16.
   for (int idx = tid; idx < NT * 4 * 64; idx += WPC * 64) {
     const int l = idx & 63;
     const int i = (idx >> 6) & 3;
     const int n = idx >> 8;
     double s = 0.0;
+    if (SPLIT) {
+      // all loads first (they are independent), then the sum in chunk order
+      const int S = gridDim.y;
+      const double *all = ws + (size_t)blockIdx.x * S * (NT * 256) + idx;
+      double v[kRouterSplitMax];
 #pragma unroll
-    for (int ww = 0; ww < WPC; ww++) s += part[ww][n][i][l];
+      for (int sp = 0; sp < kRouterSplitMax; sp++) v[sp] = sp < S ? all[(size_t)sp * (NT * 256)] : 0.0;
+#pragma unroll
+      for (int sp = 0; sp < kRouterSplitMax; sp++) s += v[sp];
+    } else {
+#pragma unroll
+      for (int ww = 0; ww < WPC; ww++) s += part[ww][n][i][l];
+    }
     const int e = 16 * n + (l & 15);
     const int tr = 4 * i + (l >> 4);
     float f = (float)s;  // run.cpp:368
@@ -120,6 +158,7 @@ __global__ __launch_bounds__(WPC * 64) void router_kernel(
     if (score && e < E && t < T && !(pos && pos[t] < 0)) score[(size_t)t * E + e] = f;
   }
   __syncthreads();
+  if (SPLIT && tid == 0) arrivals[blockIdx.x] = 0;  // for the next launch
 
   if (w != 0) return;
   // Wave 0: four lanes per token, each owning a contiguous quarter of the experts.
@@ -179,32 +218,53 @@ __global__ __launch_bounds__(WPC * 64) void router_kernel(
   *reinterpret_cast<float4 *>(topk_v + (size_t)t * kTopK) = ov;
 }
 
+// Chunks of 32 k per workgroup when a tile of 16 tokens is shared (0: no
+// sharing): batches of few tiles only, and never more than kRouterSplitMax
+// workgroups per tile.
+static int router_split_chunks(int T, int H) {
+  const int tiles = (T + 15) / 16;
+  const int kc_total = H / 32;
+  if (tiles > kRouterSplitTiles) return 0;
+  const int cps = (kc_total + kRouterSplitMax - 1) / kRouterSplitMax;
+  return cps >= kc_total ? 0 : cps;
+}
+
 template <int NT>
 static hipError_t launch_router_nt(const uint16_t *x, const int *pos, const uint16_t *wr,
                                    const float *br, int T, int H, int E, float *score, int *topk_i,
-                                   float *topk_v, hipStream_t s) {
+                                   float *topk_v, double *ws, int *arrivals, hipStream_t s) {
   const int grid = (T + 15) / 16;
+  // Register sets in flight per wave, 4 * (1 + NT) registers each, within the
+  // 128 / 256 / 512 registers a wave of a workgroup this size can have.
+  constexpr int D = NT <= 2 ? 6 : (NT <= 4 ? 4 : (NT <= 8 ? 3 : 2));
+  const int cps = ws ? router_split_chunks(T, H) : 0;
+  if (cps > 0) {
+    constexpr int WPS = NT <= 8 ? 4 : 2;  // waves of a workgroup that shares a tile
+    constexpr int DS = D < 3 ? D : 3;
+    const int S = (H / 32 + cps - 1) / cps;
+    router_kernel<NT, WPS, DS, true><<<dim3(grid, S), WPS * 64, 0, s>>>(x, pos, wr, br, T, H, E, score, topk_i,
+                                                                        topk_v, ws, arrivals, cps);
+    return hipGetLastError();
+  }
   // As many waves per workgroup (i.e. as fine a split of the reduction) as the
   // LDS for the partial sums allows (WPC * NT * 2 KB <= 64 KB): more waves per
   // SIMD hide the load latency, and small batches still occupy the SIMDs.
   constexpr int WPC = NT <= 2 ? 16 : (NT <= 4 ? 8 : (NT <= 8 ? 4 : 2));
-  // Register sets in flight per wave, 4 * (1 + NT) registers each, within the
-  // 128 / 256 / 512 registers a wave of a workgroup this size can have.
-  constexpr int D = NT <= 2 ? 6 : (NT <= 4 ? 4 : (NT <= 8 ? 3 : 2));
-  router_kernel<NT, WPC, D><<<grid, WPC * 64, 0, s>>>(x, pos, wr, br, T, H, E, score, topk_i, topk_v);
+  router_kernel<NT, WPC, D, false><<<grid, WPC * 64, 0, s>>>(x, pos, wr, br, T, H, E, score, topk_i,
+                                                             topk_v, nullptr, nullptr, 0);
   return hipGetLastError();
 }
 
 hipError_t launch_router(const uint16_t *x, const int *pos, const uint16_t *wr, const float *br, int T,
                          int H, int E, int E_pad, float *score, int *topk_i, float *topk_v,
-                         hipStream_t s) {
+                         double *ws, int *arrivals, hipStream_t s) {
   if (T <= 0) return hipSuccess;
   switch (E_pad / 16) {
-    case 1: return launch_router_nt<1>(x, pos, wr, br, T, H, E, score, topk_i, topk_v, s);
-    case 2: return launch_router_nt<2>(x, pos, wr, br, T, H, E, score, topk_i, topk_v, s);
-    case 4: return launch_router_nt<4>(x, pos, wr, br, T, H, E, score, topk_i, topk_v, s);
-    case 8: return launch_router_nt<8>(x, pos, wr, br, T, H, E, score, topk_i, topk_v, s);
-    case 16: return launch_router_nt<16>(x, pos, wr, br, T, H, E, score, topk_i, topk_v, s);
+    case 1: return launch_router_nt<1>(x, pos, wr, br, T, H, E, score, topk_i, topk_v, ws, arrivals, s);
+    case 2: return launch_router_nt<2>(x, pos, wr, br, T, H, E, score, topk_i, topk_v, ws, arrivals, s);
+    case 4: return launch_router_nt<4>(x, pos, wr, br, T, H, E, score, topk_i, topk_v, ws, arrivals, s);
+    case 8: return launch_router_nt<8>(x, pos, wr, br, T, H, E, score, topk_i, topk_v, ws, arrivals, s);
+    case 16: return launch_router_nt<16>(x, pos, wr, br, T, H, E, score, topk_i, topk_v, ws, arrivals, s);
     default: return hipErrorInvalidValue;
   }
 }

@@ -271,11 +271,12 @@ def test_all_tokens_on_four_experts_and_tiny_batches(c2):
         check_outputs(R, L2, x, None, np.arange(T))
 
 
-@pytest.mark.parametrize("T", [16, 17, 64, 65, 256, 257])
+@pytest.mark.parametrize("T", [16, 17, 64, 65, 128, 129, 256, 257])
 def test_batch_size_boundaries(c2, T):
     """Either side of the sizes at which the library changes its plan: up to 64
     rows per expert the GEMMs run in their small-batch configuration and gate_up
-    reads the token rows itself, up to 256 tokens the dispatch is one workgroup.
+    reads the token rows itself, up to 128 tokens several workgroups share a
+    router tile, up to 256 tokens the dispatch is one workgroup.
     moe_forward bounds the rows per expert by T, moe_experts (whose ids come from
     the caller) by 4 T, so between 17 and 64 tokens the two entry points take
     different configurations for the same work: same bits required."""
@@ -415,11 +416,13 @@ def test_ffn_block_in_place(c2, T):
         m2.block_forward(0, dx, None, 16)
 
 
-def test_forward_replays_from_a_hip_graph(c2):
+@pytest.mark.parametrize("T", [1500, 48])
+def test_forward_replays_from_a_hip_graph(c2, T):
     """moe_forward allocates nothing, never synchronises and clears its buffers
     with kernels, so a caller may capture it.  Three replays, with eager calls
     and synchronisations of the program's own in between, must each reproduce the
-    eager result bit for bit."""
+    eager result bit for bit.  48 tokens take the small-batch kernels (the
+    arrival counters of the shared router tiles are reset by the kernel itself)."""
     import ctypes as C
     hip = C.CDLL("libamdhip64.so")
 
@@ -427,7 +430,6 @@ def test_forward_replays_from_a_hip_graph(c2):
         assert rc == 0, f"HIP call failed with {rc}"
 
     sh, L, m = c2
-    T = 1500
     x = L["x"][:T]
     dx = abi.DevBuf.from_numpy(synth.to_bf16_bits(x))
     dout, dref = abi.DevBuf(T * sh.hidden * 4), abi.DevBuf(T * sh.hidden * 4)
