@@ -22,7 +22,8 @@ SYMBOLS = [
     "moe_create", "moe_destroy", "moe_upload_layer", "moe_upload_layer_mxfp4", "moe_upload_norm",
     "moe_forward", "moe_block_forward",
     "moe_router",
-    "moe_dispatch", "moe_get_dispatch", "moe_experts", "moe_profile_enable",
+    "moe_dispatch", "moe_get_dispatch", "moe_experts", "moe_expert_gemms", "moe_combine",
+    "moe_profile_enable",
     "moe_profile_read", "moe_weight_bytes", "moe_workspace_bytes", "moe_last_error",
     "moe_version", "moe_dev_alloc", "moe_dev_free", "moe_dev_upload", "moe_dev_download",
     "moe_dev_memset", "moe_dev_sync", "moe_dev_count", "moe_time_forward",
@@ -63,6 +64,8 @@ def lib() -> C.CDLL:
         L.moe_dispatch.argtypes = [vp, vp, vp, ci, vp]
         L.moe_get_dispatch.argtypes = [vp, vp, vp, ci, vp]
         L.moe_experts.argtypes = [vp, ci, vp, vp, vp, vp, ci, vp, ci, vp]
+        L.moe_expert_gemms.argtypes = [vp, ci, vp, ci, vp]
+        L.moe_combine.argtypes = [vp, vp, vp, ci, vp, ci, vp]
         L.moe_profile_enable.argtypes = [vp, ci]
         L.moe_profile_read.argtypes = [vp, C.POINTER(cf), C.POINTER(ci)]
         L.moe_weight_bytes.argtypes = [vp]
@@ -201,6 +204,13 @@ class Moe:
     def experts(self, layer, x, pos, topk_i, topk_v, n_tokens, out, accumulate=False, stream=None):
         check(lib().moe_experts(self.h, layer, _p(x), _p(pos), _p(topk_i), _p(topk_v), n_tokens,
                                 _p(out), 1 if accumulate else 0, stream))
+
+    def expert_gemms(self, layer, x, n_tokens, stream=None):
+        check(lib().moe_expert_gemms(self.h, layer, _p(x), n_tokens, stream))
+
+    def combine(self, topk_v, pos, n_tokens, out, accumulate=False, stream=None):
+        check(lib().moe_combine(self.h, _p(topk_v), _p(pos), n_tokens, _p(out),
+                                1 if accumulate else 0, stream))
 
     def profile_enable(self, n_calls):
         check(lib().moe_profile_enable(self.h, n_calls))

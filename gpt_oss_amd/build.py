@@ -8,7 +8,6 @@ import sys
 PKG = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(PKG, "csrc")
 LIB = os.path.join(PKG, "libmi355_moe.so")
-PROBE = os.path.join(PKG, "ingest_probe.exe")
 SOURCES = ["moe_api.hip", "pack.hip", "router.hip", "dispatch.hip", "gemm.hip", "norm.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
@@ -19,32 +18,30 @@ FLAGS = [
 ]
 
 
+def _compile(src: str, verbose: bool, extra: list[str] | None) -> str:
+    obj = os.path.join(CSRC, src.replace(".hip", ".o"))
+    cmd = [c for c in [HIPCC, *FLAGS, "-c", os.path.join(CSRC, src), "-o", obj] if c != "-shared"]
+    cmd += extra or []
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    err = "\n".join(l for l in r.stderr.splitlines() if "packed-fp32-ops" not in l)
+    if r.returncode != 0:
+        raise RuntimeError(f"hipcc failed on {src}:\n{err}")
+    if verbose and err.strip():
+        print(err, file=sys.stderr)
+    return obj
+
+
 def build_lib(verbose: bool = True, extra: list[str] | None = None) -> str:
-    objs = []
-    for src in SOURCES:
-        obj = os.path.join(CSRC, src.replace(".hip", ".o"))
-        cmd = [HIPCC, *FLAGS[:-0 or None], "-c", os.path.join(CSRC, src), "-o", obj]
-        cmd = [c for c in cmd if c != "-shared"] + (extra or [])
-        if verbose:
-            print(" ".join(cmd), flush=True)
-        r = subprocess.run(cmd, capture_output=True, text=True)
-        err = "\n".join(l for l in r.stderr.splitlines() if "packed-fp32-ops" not in l)
-        if r.returncode != 0:
-            raise RuntimeError(f"hipcc failed on {src}:\n{err}")
-        if verbose and err.strip():
-            print(err, file=sys.stderr)
-        objs.append(obj)
+    # one hipcc per source file, side by side (the GEMM's template instances dominate)
+    from concurrent.futures import ThreadPoolExecutor
+    with ThreadPoolExecutor(max_workers=min(len(SOURCES), os.cpu_count() or 1, 8)) as ex:
+        objs = list(ex.map(lambda src: _compile(src, verbose, extra), SOURCES))
     cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", *objs, "-o", LIB]
     if verbose:
         print(" ".join(cmd), flush=True)
     subprocess.check_call(cmd)
-    # stand-alone measurement tool (streaming ceilings, counter calibration)
-    cmd = [HIPCC, "--offload-arch=gfx950", "-O3", os.path.join(CSRC, "ingest_probe.hip"), "-o", PROBE]
-    if verbose:
-        print(" ".join(cmd), flush=True)
-    r = subprocess.run(cmd, capture_output=True, text=True)
-    if r.returncode != 0:
-        raise RuntimeError(f"hipcc failed on ingest_probe.hip:\n{r.stderr}")
     return LIB
 
 

@@ -431,10 +431,10 @@ __global__ __launch_bounds__(256) void gather_rows_kernel(const uint16_t *__rest
                                                          const int *__restrict__ rowmap,
                                                          const int *__restrict__ totals,
                                                          uint4 *__restrict__ xg, int H) {
-  const int rb = blockIdx.y;
+  const int rb = blockIdx.x;  // the x dimension of a grid has room for any batch the handle accepts
   if (rb * kRowBlock >= totals[1]) return;
   const int lane = threadIdx.x & 63;
-  const int grp = blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int grp = blockIdx.y * 4 + (threadIdx.x >> 6);
   const int kb_total = H / kFragK;
   if (grp * 4 >= kb_total) return;
   const int a = rowmap[rb * kRowBlock + (lane & 31)];
@@ -531,7 +531,7 @@ hipError_t launch_gather(const uint16_t *x, const DispatchBuffers &d, uint16_t *
                          int rb_cap, hipStream_t s) {
   (void)T;
   const int groups = H / 64;
-  dim3 grid((groups + 3) / 4, rb_cap);
+  dim3 grid(rb_cap, (groups + 3) / 4);
   gather_rows_kernel<<<grid, 256, 0, s>>>(x, d.rowmap, d.totals, reinterpret_cast<uint4 *>(xg), H);
   return hipGetLastError();
 }

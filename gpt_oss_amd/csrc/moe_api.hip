@@ -14,16 +14,21 @@
 using namespace moe;
 
 namespace {
-
 thread_local char g_err[512] = "";
+}
 
-int fail(int code, const char *fmt, ...) {
+// Records the text of a failure for moe_last_error() and returns `code`.
+int moe::set_error(int code, const char *fmt, ...) {
   va_list ap;
   va_start(ap, fmt);
   vsnprintf(g_err, sizeof(g_err), fmt, ap);
   va_end(ap);
   return code;
 }
+
+namespace {
+
+#define fail moe::set_error
 
 #define HIP_TRY(call)                                                                       \
   do {                                                                                      \
@@ -54,13 +59,12 @@ struct moe_handle {
   // routing produced by the router stage (or copied from the caller)
   int *topk_i = nullptr;
   float *topk_v = nullptr;
-  double *router_ws = nullptr;     // sums of the router's shared-tile form
-  int *router_arrivals = nullptr;  // its arrival counters, zero between launches
   // dispatch
   DispatchBuffers disp{};
   int a_cap = 0;      // max assignments
   int a_pad_cap = 0;  // max padded rows
   int n_blk_cap = 0;
+  int disp_tokens = -1;  // batch of the last moe_dispatch (stage-level calls), -1: none
   // expert pipeline
   uint16_t *xg = nullptr;   // gathered rows, bf16 fragments
   uint16_t *act = nullptr;  // SwiGLU output, bf16 fragments
@@ -127,18 +131,16 @@ inline int down_col_tiles(const moe_config &c) {
   return (c.hidden / kRowBlock + kGemmTileNb - 1) / kGemmTileNb;
 }
 
-// out != nullptr: out (+)= layer(x), fp32.  Otherwise resid (bf16, in place) += layer(x).
+// Stages 3-5 on the plan of the last dispatch: gather (large batches), gate_up
+// GEMM with the SwiGLU, down GEMM.  Leaves the per-assignment rows in h->y.
 // max_rows: no expert is given more rows than this (T when the ids of a token are distinct).
-int run_experts(moe_handle *h, int layer, const uint16_t *x, const int *pos, const int *topk_i,
-                const float *topk_v, int T, int max_rows, float *out, int accumulate, hipStream_t s,
-                StageTimer &tm, uint16_t *resid = nullptr) {
+int run_gemms(moe_handle *h, int layer, const uint16_t *x, int T, int max_rows, hipStream_t s,
+              StageTimer &tm) {
   const moe_config &c = h->cfg;
   const LayerWeights &lw = h->layers[layer];
   const int A = T * kTopK;
   const int mt_cap = A / kTileRows + c.experts;
   const int rb_cap = (A + kTileGran * c.experts + kRowBlock - 1) / kRowBlock;
-  HIP_TRY(tm.mark(MOE_STAGE_DISPATCH));
-  HIP_TRY(launch_dispatch(topk_i, pos, T, c.experts, gate_up_col_tiles(c), down_col_tiles(c), h->disp, s));
   HIP_TRY(tm.mark(MOE_STAGE_GATHER));
   if (!gate_up_gathers(max_rows)) HIP_TRY(launch_gather(x, h->disp, h->xg, T, c.hidden, rb_cap, s));
   HIP_TRY(tm.mark(MOE_STAGE_GATE_UP));
@@ -147,14 +149,34 @@ int run_experts(moe_handle *h, int layer, const uint16_t *x, const int *pos, con
   HIP_TRY(tm.mark(MOE_STAGE_DOWN));
   HIP_TRY(launch_down(h->act, lw.w2q ? static_cast<const void *>(lw.w2q) : lw.w2, lw.w2s, lw.b2,
                       h->disp, h->y, c.hidden, c.inter, mt_cap, max_rows, s));
+  return MOE_OK;
+}
+
+// Stage 6: out != nullptr: out (+)= sum_k w[t,k] * y[row of (t,k)], fp32.
+// Otherwise resid (bf16, in place) += that sum.
+int run_combine(moe_handle *h, const float *topk_v, const int *pos, int T, float *out, int accumulate,
+                uint16_t *resid, hipStream_t s, StageTimer &tm) {
   HIP_TRY(tm.mark(MOE_STAGE_COMBINE));
   if (out) {
-    HIP_TRY(launch_combine(h->y, h->disp.inv, topk_v, pos, out, T, c.hidden, accumulate, s));
+    HIP_TRY(launch_combine(h->y, h->disp.inv, topk_v, pos, out, T, h->cfg.hidden, accumulate, s));
   } else {
-    HIP_TRY(launch_combine_residual(h->y, h->disp.inv, topk_v, pos, resid, T, c.hidden, s));
+    HIP_TRY(launch_combine_residual(h->y, h->disp.inv, topk_v, pos, resid, T, h->cfg.hidden, s));
   }
   HIP_TRY(tm.mark(MOE_NUM_STAGES));
   return MOE_OK;
+}
+
+// Stages 2-6.
+int run_experts(moe_handle *h, int layer, const uint16_t *x, const int *pos, const int *topk_i,
+                const float *topk_v, int T, int max_rows, float *out, int accumulate, hipStream_t s,
+                StageTimer &tm, uint16_t *resid = nullptr) {
+  const moe_config &c = h->cfg;
+  HIP_TRY(tm.mark(MOE_STAGE_DISPATCH));
+  HIP_TRY(launch_dispatch(topk_i, pos, T, c.experts, gate_up_col_tiles(c), down_col_tiles(c), h->disp, s));
+  h->disp_tokens = -1;  // the plan now belongs to this call, not to a moe_dispatch
+  int rc = run_gemms(h, layer, x, T, max_rows, s, tm);
+  if (rc != MOE_OK) return rc;
+  return run_combine(h, topk_v, pos, T, out, accumulate, resid, s, tm);
 }
 
 }  // namespace
@@ -201,8 +223,6 @@ int moe_create(const moe_config *cfg, moe_handle **out) {
   if (rc == MOE_OK) rc = dev_alloc(h, &(ptr), (count), true)
   ALLOC(h->topk_i, (size_t)h->a_cap);
   ALLOC(h->topk_v, (size_t)h->a_cap);
-  ALLOC(h->router_ws, (size_t)kRouterSplitTiles * kRouterSplitMax * h->E_pad * 16);
-  ALLOC(h->router_arrivals, (size_t)kRouterSplitTiles);
   ALLOC(h->disp.blk_counts, (size_t)h->n_blk_cap * E);
   ALLOC(h->disp.offsets, (size_t)E + 1);
   ALLOC(h->disp.perm, (size_t)h->a_cap);
@@ -222,10 +242,6 @@ int moe_create(const moe_config *cfg, moe_handle **out) {
   ALLOC(h->y, (size_t)h->a_pad_cap * H);
 #undef ALLOC
   h->disp.a_pad_cap = h->a_pad_cap;
-  if (rc == MOE_OK) {
-    const hipError_t e0 = hipMemset(h->router_arrivals, 0, kRouterSplitTiles * sizeof(int));
-    if (e0 != hipSuccess) rc = fail(MOE_ERR_HIP, "hipMemset failed: %s", hipGetErrorString(e0));
-  }
   if (rc != MOE_OK) {
     moe_destroy(h);
     return rc;
@@ -245,7 +261,6 @@ int moe_destroy(moe_handle *h) {
     (void)hipFree(lw.w1q); (void)hipFree(lw.w1s); (void)hipFree(lw.w2q); (void)hipFree(lw.w2s);
   }
   (void)hipFree(h->topk_i); (void)hipFree(h->topk_v);
-  (void)hipFree(h->router_ws); (void)hipFree(h->router_arrivals);
   (void)hipFree(h->disp.blk_counts); (void)hipFree(h->disp.offsets); (void)hipFree(h->disp.perm);
   (void)hipFree(h->disp.rowmap); (void)hipFree(h->disp.inv); (void)hipFree(h->disp.info); (void)hipFree(h->disp.totals);
   (void)hipFree(h->disp.tiles_gate_up); (void)hipFree(h->disp.tiles_down);
@@ -269,6 +284,9 @@ int upload_layer(moe_handle *h, int layer, const float *w_router, const float *b
                  const float *b_mlp1, const float *b_mlp2, const ExpertSource &src) {
   const int E = h->cfg.experts, H = h->cfg.hidden, IM = h->cfg.inter, E_pad = h->E_pad;
   LayerWeights &lw = h->layers[layer];
+  // not usable until this upload has gone through: a failure below leaves the
+  // layer without weights rather than with freed or half-written ones
+  lw.uploaded = false;
   int rc = MOE_OK;
 #define ALLOCW(ptr, count)                                             \
   if (rc == MOE_OK && !(ptr)) rc = dev_alloc(h, &(ptr), (count), false)
@@ -286,7 +304,7 @@ int upload_layer(moe_handle *h, int layer, const float *w_router, const float *b
     lw.w1s = lw.w2s = nullptr;
   }
   ALLOCW(lw.wr, (size_t)E_pad * H);
-  ALLOCW(lw.br, (size_t)E_pad);
+  ALLOCW(lw.br, (size_t)E_pad + 2);
   ALLOCW(lw.b1g, (size_t)E * IM);
   ALLOCW(lw.b1u, (size_t)E * IM);
   ALLOCW(lw.b2, (size_t)E * H);
@@ -317,6 +335,7 @@ int upload_layer(moe_handle *h, int layer, const float *w_router, const float *b
     HIP_TRY(hipMemcpy(stage, w_router, (size_t)E * H * sizeof(float), hipMemcpyHostToDevice));
     HIP_TRY(hipMemcpy(stage_b, b_router, (size_t)E * sizeof(float), hipMemcpyHostToDevice));
     HIP_TRY(launch_pack_router(stage, stage_b, lw.wr, lw.br, E, E_pad, H, nullptr));
+    HIP_TRY(launch_router_stats(stage, stage_b, E, H, lw.br + E_pad, nullptr));
     HIP_TRY(hipDeviceSynchronize());
     HIP_TRY(hipMemcpy(stage_b, b_mlp1, (size_t)E * 2 * IM * sizeof(float), hipMemcpyHostToDevice));
     HIP_TRY(launch_pack_bias(stage_b, lw.b1g, lw.b1u, E * 2 * IM, true, nullptr));
@@ -406,9 +425,8 @@ int moe_router(moe_handle *h, int layer, const uint16_t *x, const int *pos, int 
   if (n_tokens > 0 && !topk_v) return fail(MOE_ERR_BAD_ARG, "null device pointer");
   if (n_tokens == 0) return MOE_OK;
   const LayerWeights &lw = h->layers[layer];
-  HIP_TRY(launch_router(x, pos, lw.wr, lw.br, n_tokens, h->cfg.hidden, h->cfg.experts, h->E_pad,
-                        score, topk_i, topk_v, h->router_ws, h->router_arrivals,
-                        static_cast<hipStream_t>(stream)));
+  HIP_TRY(launch_router(x, pos, lw.wr, lw.br, lw.br + h->E_pad, n_tokens, h->cfg.hidden, h->cfg.experts,
+                        h->E_pad, score, topk_i, topk_v, static_cast<hipStream_t>(stream)));
   return MOE_OK;
 }
 
@@ -420,6 +438,7 @@ int moe_dispatch(moe_handle *h, const int *topk_i, const int *pos, int n_tokens,
   if (n_tokens > 0 && !topk_i) return fail(MOE_ERR_BAD_ARG, "null device pointer");
   HIP_TRY(launch_dispatch(topk_i, pos, n_tokens, h->cfg.experts, gate_up_col_tiles(h->cfg),
                           down_col_tiles(h->cfg), h->disp, static_cast<hipStream_t>(stream)));
+  h->disp_tokens = n_tokens;
   return MOE_OK;
 }
 
@@ -452,6 +471,34 @@ int moe_experts(moe_handle *h, int layer, const uint16_t *x, const int *pos, con
   return rc;
 }
 
+int moe_expert_gemms(moe_handle *h, int layer, const uint16_t *x, int n_tokens, void *stream) {
+  int rc = check_forward_args(h, layer, x, n_tokens, x);
+  if (rc != MOE_OK) return rc;
+  if (h->disp_tokens != n_tokens)
+    return fail(MOE_ERR_STATE, "moe_expert_gemms(%d tokens) needs a moe_dispatch of the same batch first (last: %d)",
+                n_tokens, h->disp_tokens);
+  if (n_tokens == 0) return MOE_OK;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  StageTimer tm(h, nullptr);  // stage-level calls are not timed
+  tm.ev = nullptr;
+  // the ids of a moe_dispatch come from outside and may name an expert in several slots of a token
+  return run_gemms(h, layer, x, n_tokens, n_tokens * kTopK, s, tm);
+}
+
+int moe_combine(moe_handle *h, const float *topk_v, const int *pos, int n_tokens, float *out,
+                int accumulate, void *stream) {
+  if (!h) return fail(MOE_ERR_BAD_ARG, "null handle");
+  if (n_tokens < 0) return fail(MOE_ERR_BAD_ARG, "n_tokens %d is negative", n_tokens);
+  if (h->disp_tokens != n_tokens)
+    return fail(MOE_ERR_STATE, "moe_combine(%d tokens) needs moe_dispatch and moe_expert_gemms of the same batch first (last: %d)",
+                n_tokens, h->disp_tokens);
+  if (n_tokens == 0) return MOE_OK;
+  if (!topk_v || !out) return fail(MOE_ERR_BAD_ARG, "null device pointer");
+  StageTimer tm(h, nullptr);
+  tm.ev = nullptr;
+  return run_combine(h, topk_v, pos, n_tokens, out, accumulate, nullptr, static_cast<hipStream_t>(stream), tm);
+}
+
 int moe_forward(moe_handle *h, int layer, const uint16_t *x, const int *pos, int n_tokens,
                 float *out, int accumulate, void *stream) {
   int rc = check_forward_args(h, layer, x, n_tokens, out);
@@ -461,8 +508,8 @@ int moe_forward(moe_handle *h, int layer, const uint16_t *x, const int *pos, int
   const LayerWeights &lw = h->layers[layer];
   StageTimer tm(h, s);
   HIP_TRY(tm.mark(MOE_STAGE_ROUTER));
-  HIP_TRY(launch_router(x, pos, lw.wr, lw.br, n_tokens, h->cfg.hidden, h->cfg.experts, h->E_pad,
-                        nullptr, h->topk_i, h->topk_v, h->router_ws, h->router_arrivals, s));
+  HIP_TRY(launch_router(x, pos, lw.wr, lw.br, lw.br + h->E_pad, n_tokens, h->cfg.hidden, h->cfg.experts,
+                        h->E_pad, nullptr, h->topk_i, h->topk_v, s));
   rc = run_experts(h, layer, x, pos, h->topk_i, h->topk_v, n_tokens, n_tokens, out, accumulate, s, tm);
   if (rc == MOE_OK) tm.done();
   return rc;
@@ -503,8 +550,8 @@ int moe_block_forward(moe_handle *h, int layer, uint16_t *x, const int *pos, int
   StageTimer tm(h, s);
   HIP_TRY(tm.mark(MOE_STAGE_ROUTER));  // the norm is counted with the router stage
   HIP_TRY(launch_rmsnorm(x, lw.rms_w, pos, h->t_norm, n_tokens, h->cfg.hidden, s));
-  HIP_TRY(launch_router(h->t_norm, pos, lw.wr, lw.br, n_tokens, h->cfg.hidden, h->cfg.experts,
-                        h->E_pad, nullptr, h->topk_i, h->topk_v, h->router_ws, h->router_arrivals, s));
+  HIP_TRY(launch_router(h->t_norm, pos, lw.wr, lw.br, lw.br + h->E_pad, n_tokens, h->cfg.hidden,
+                        h->cfg.experts, h->E_pad, nullptr, h->topk_i, h->topk_v, s));
   rc = run_experts(h, layer, h->t_norm, pos, h->topk_i, h->topk_v, n_tokens, n_tokens, nullptr, 0, s, tm,
                    x);
   if (rc == MOE_OK) tm.done();
@@ -517,7 +564,15 @@ int moe_profile_enable(moe_handle *h, int n_calls) {
     return fail(MOE_ERR_BAD_ARG, "n_calls %d outside [0,%d]", n_calls, kMaxProfileCalls);
   if (h->events.empty()) {
     h->events.resize((size_t)kMaxProfileCalls * (MOE_NUM_STAGES + 1), nullptr);
-    for (auto &ev : h->events) HIP_TRY(hipEventCreate(&ev));
+    for (auto &ev : h->events) {
+      const hipError_t e = hipEventCreate(&ev);
+      if (e != hipSuccess) {  // all events or none: later calls record into every one of them
+        for (hipEvent_t made : h->events)
+          if (made) (void)hipEventDestroy(made);
+        h->events.clear();
+        return fail(MOE_ERR_HIP, "hipEventCreate failed: %s", hipGetErrorString(e));
+      }
+    }
   }
   h->prof_armed = n_calls;
   h->prof_recorded = 0;

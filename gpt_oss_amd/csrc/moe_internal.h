@@ -9,6 +9,10 @@
 
 namespace moe {
 
+// Records the text of a failure for moe_last_error() on the calling thread and
+// returns `code` (defined with the C-ABI's host side).
+int set_error(int code, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
+
 // float -> bf16 bits, round to nearest even; a NaN stays a NaN
 // (/opt/rocm/include/hip/amd_detail/amd_hip_bfloat16.h:96-131).
 __device__ __forceinline__ uint16_t f32_to_bf16_rne(float f) {
@@ -76,8 +80,8 @@ struct TileDesc {
 };
 
 struct LayerWeights {
-  uint16_t *wr = nullptr;  // router weight, bf16 in the operand order of the f64 MFMA
-  float *br = nullptr;     // router bias, padded experts = -inf
+  uint16_t *wr = nullptr;  // router weight, bf16 in the operand order of v_mfma_f32_16x16x32_bf16
+  float *br = nullptr;     // router bias [E_pad] (padded experts = -inf), then the two floats of rstat
   uint16_t *w1 = nullptr;  // gate_up weight, bf16 MFMA fragments, gate/up blocks paired
   float *b1g = nullptr;    // gate bias [E, IM]
   float *b1u = nullptr;    // up bias   [E, IM]
@@ -103,15 +107,14 @@ hipError_t launch_pack_fp4(const uint8_t *blocks, const uint8_t *scales, uint8_t
 hipError_t launch_pack_bias(const float *src, float *dst_a, float *dst_b, int n, bool deinterleave,
                             hipStream_t s);
 
-// ws / arrivals: workspace of the router's shared-tile form (kRouterSplitTiles *
-// kRouterSplitMax * E_pad * 16 doubles; kRouterSplitTiles ints, zero before the
-// first launch and left zero by every launch); ws == nullptr keeps one
-// workgroup per 16 tokens.
-constexpr int kRouterSplitTiles = 8;   // batches of at most this many tiles of 16 tokens share tiles
-constexpr int kRouterSplitMax = 16;    // workgroups per shared tile, at most
-hipError_t launch_router(const uint16_t *x, const int *pos, const uint16_t *wr, const float *br, int T,
-                         int H, int E, int E_pad, float *score, int *topk_i, float *topk_v,
-                         double *ws, int *arrivals, hipStream_t s);
+// rstat: two floats written by launch_router_stats at upload (largest 2-norm of
+// an expert's router weights, largest bias magnitude), the inputs of the error
+// bound that decides which tokens need exact fp64 logits.
+hipError_t launch_router_stats(const float *w_src, const float *b_src, int E, int H, float *rstat,
+                               hipStream_t s);
+hipError_t launch_router(const uint16_t *x, const int *pos, const uint16_t *wr, const float *br,
+                         const float *rstat, int T, int H, int E, int E_pad, float *score, int *topk_i,
+                         float *topk_v, hipStream_t s);
 
 struct DispatchBuffers {
   int *blk_counts;    // [n_blk, E]

@@ -85,13 +85,11 @@ __global__ void pack_fp4_kernel(const uint8_t *__restrict__ blocks, const uint8_
   }
 }
 
-// Router weight in the operand order of v_mfma_f64_16x16x4_f64, kept as bf16
-// (the kernel widens to f64 on the fly: a quarter of the bytes of an f64 copy,
-// and the router is otherwise bound by streaming this matrix through every CU).
-// Order [expert block of 16][k chunk of 32][lane][s], s = 0..7: lane l holds
-// expert 16*nb + (l % 16) and k = 32*kc + 8*(l / 16) + s.  The s-th MFMA of a
-// chunk multiplies these with the s-th of 8 consecutive activations a lane loaded.
-// Experts beyond E are zero weight with bias -inf, so they are never selected.
+// Router weight as bf16 in the operand order of v_mfma_f32_16x16x32_bf16:
+// [expert block of 16][k chunk of 32][lane][s], s = 0..7: lane l holds expert
+// 16*nb + (l % 16) and k = 32*kc + 8*(l / 16) + s, the same split of a chunk's
+// k over the lanes as the activations are loaded with.  Experts beyond E are
+// zero weight with bias -inf; the selection skips them by index.
 __global__ void pack_router_kernel(const float *__restrict__ w, const float *__restrict__ b,
                                    uint16_t *__restrict__ wr, float *__restrict__ br, int E,
                                    int E_pad, int H) {

@@ -1,270 +1,398 @@
 // Router: logits = x * Wr^T + br, top-4 with ties to the lower expert id,
 // softmax over the four selected logits.  Replaces matmul_router_kernel
 // (matmul/matmul.cpp:945-1019) and fused_topk_softmax_batch_kernel
-// (utility/utility.cpp:273-365); the arithmetic follows the reference's CPU path
-// (run.cpp:356-369 matmul, :388-421 topk, :336-354 softmax) so that the expert
-// ids are reproduced exactly:
-//   * products of two bf16 values are exact in fp32; they are accumulated in
-//     fp64 on the matrix cores (v_mfma_f64_16x16x4_f64), as run.cpp:363-367
-//     accumulates float products in a double; the sum is rounded to float once
-//     and the bias is added in float (run.cpp:669-671);
-//   * the top-4 comparison is (value descending, index ascending);
-//   * the softmax keeps the sum in double and divides in double.
+// (utility/utility.cpp:273-365).  The expert ids must be those of the
+// reference's CPU path (run.cpp:356-369 matmul: float products accumulated in a
+// double, rounded to float once; :669-671 bias added in float; :388-421 top-k;
+// :336-354 softmax), bit for bit.
+//
+// Two passes in one kernel:
+//   1. All logits on the bf16 matrix cores (v_mfma_f32_16x16x32_bf16).  The
+//      products are exact; the fp32 accumulation inside the matrix core is not,
+//      so a wave hands its fp32 sums over to fp64 accumulators every kFlush
+//      MFMAs.  That bounds the error of a logit by kGamma * sum_k |x_k w_ek|
+//      <= kGamma * |x| * |w_e| (Cauchy-Schwarz; |x|^2 comes out of one more
+//      MFMA per chunk, x times its own transpose, and max_e |w_e| is computed
+//      at upload).
+//   2. A token whose five best logits are further apart than twice that bound
+//      is decided: ids, order and (to about 1e-7) weights are those of the
+//      exact arithmetic.  For any other token the experts that can still reach
+//      the top four -- those within the bound of the fourth best -- get their
+//      logit recomputed exactly: float products (exact for bf16 factors)
+//      summed in fp64, rounded to float once, bias added in float, which is the
+//      arithmetic of run.cpp:363-369 up to the order of the fp64 additions.
+//      An expert outside that set is below four experts by more than the two
+//      error bounds, so it cannot be among the exact top four; inside the set
+//      all values are exact, so the selection (value descending, index
+//      ascending) is the reference's.
+// At the benchmark shapes a few per cent of the tokens take the second pass,
+// with four to six experts each, instead of every token paying fp64 for every
+// expert.
 #include "moe_internal.h"
 
 namespace moe {
 
-typedef double f64x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
 
-// 8 bf16 -> 8 doubles (exact).
-__device__ __forceinline__ void widen8(const uint4 v, double (&d)[8]) {
-  d[0] = (double)__uint_as_float(v.x << 16);
-  d[1] = (double)__uint_as_float(v.x & 0xffff0000u);
-  d[2] = (double)__uint_as_float(v.y << 16);
-  d[3] = (double)__uint_as_float(v.y & 0xffff0000u);
-  d[4] = (double)__uint_as_float(v.z << 16);
-  d[5] = (double)__uint_as_float(v.z & 0xffff0000u);
-  d[6] = (double)__uint_as_float(v.w << 16);
-  d[7] = (double)__uint_as_float(v.w & 0xffff0000u);
-}
+constexpr int kFlush = 4;  // MFMAs (of 32 k) between two hand-overs to fp64
+// Error of one fp32 chain of kFlush MFMAs started from zero, relative to the
+// sum of the magnitudes of its 32 * kFlush products: every one of its
+// 33 * kFlush additions is taken to lose at most 2^-23 of the running
+// magnitude (covers truncation as well as rounding), and the result is doubled.
+constexpr float kGamma = 2.0f * 33.0f * kFlush * 1.1920929e-7f;
+constexpr int kNone = 0x7fffffff;
 
-// One workgroup = 16 tokens x all experts.  Its WPC waves split the reduction
-// dimension in chunks of 32 (wave w takes chunks w, w+WPC, ...), each wave
-// keeps NT 16x16 accumulators, and the partial sums are added in wave order
-// through LDS.  NT = E_pad / 16.
-//
-// SPLIT (small batches: a handful of workgroups would otherwise carry all the
-// fp64 MFMAs on as many CUs, 20 us whatever the batch): gridDim.y workgroups
-// share a tile of 16 tokens, each taking `cps` consecutive chunks.  They leave
-// their sums in `ws`; the one that arrives last (a counter per tile) adds them
-// up in the order of the chunks -- the same sum whichever arrives last -- and
-// selects.  No workgroup waits for another.
-template <int NT, int WPC, int D, bool SPLIT>
-__global__ __launch_bounds__(WPC * 64) void router_kernel(
-    const uint16_t *__restrict__ x, const int *__restrict__ pos, const uint16_t *__restrict__ wr,
-    const float *__restrict__ br, int T, int H, int E, float *__restrict__ score,
-    int *__restrict__ topk_i, float *__restrict__ topk_v, double *ws, int *arrivals, int cps) {
-  constexpr int E_pad = NT * 16;
-  __shared__ double part[WPC][NT][4][64];  // [wave][expert block][reg][lane]
-  __shared__ float logits[16][E_pad + 1];
-  __shared__ int is_last;
-
-  const int tid = threadIdx.x;
-  const int lane = tid & 63;
-  const int w = tid >> 6;
-  const int tok0 = blockIdx.x * 16;
-  const int row = lane & 15;  // token within the tile (A-operand row)
-  const int g = lane >> 4;    // which 8 of the chunk's 32 k this lane holds
-  const int t_ld = min(tok0 + row, T - 1);
-  const int kc_total = H / 32;
-  const int c_begin = SPLIT ? (int)blockIdx.y * cps : 0;
-  const int c_end = SPLIT ? min(c_begin + cps, kc_total) : kc_total;
-
-  f64x4 acc[NT];
+// Top-NSEL of a token's logits held by four lanes (lane q owns experts
+// q*PER .. q*PER+PER-1), by the rule of the reference's CPU top-k under a stable
+// sort: value descending, index ascending; a candidate replaces the incumbent
+// (the one with the lower index) only if it compares strictly greater, so a
+// NaN neither wins nor loses a comparison and a row of NaNs selects 0, 1, 2, 3.
+// Experts >= E are never selected.  All four lanes end with the same result.
+template <int PER, int NSEL>
+__device__ __forceinline__ void select_top(const float (&v)[PER], int q, int E, float (&sel_v)[NSEL],
+                                           int (&sel_i)[NSEL]) {
+  unsigned long long taken = 0;
 #pragma unroll
-  for (int n = 0; n < NT; n++) acc[n] = f64x4{0.0, 0.0, 0.0, 0.0};
-
-  // The wave's loads run D chunks ahead of its MFMAs (a ring of D register
-  // sets): with few waves per SIMD nothing else covers their latency, and a
-  // small batch is a handful of workgroups whose time is the chain of these
-  // round trips.  Past the end the ring re-loads the last chunk and drops it.
-  const uint16_t *xrow = x + (size_t)t_ld * H + g * 8;
-  const uint16_t *wlane = wr + (size_t)lane * 8;
-  uint4 xs[D], wq[D][NT];
-  auto load = [&](int d, int c) {
-    const int cc = min(c, c_end - 1);
-    xs[d] = *reinterpret_cast<const uint4 *>(xrow + cc * 32);
-#pragma unroll
-    for (int n = 0; n < NT; n++)
-      wq[d][n] = *reinterpret_cast<const uint4 *>(wlane + ((size_t)n * kc_total + cc) * 512);
-  };
-#pragma unroll
-  for (int d = 0; d < D; d++) load(d, c_begin + w + d * WPC);
-  for (int c0 = c_begin + w; c0 < c_end; c0 += D * WPC) {
-#pragma unroll
-    for (int d = 0; d < D; d++) {
-      const int c = c0 + d * WPC;
-      if (c < c_end) {  // the same for the whole wave
-        double xd[8];
-        widen8(xs[d], xd);
-        // Two accumulators are advanced alternately so that back-to-back MFMAs do
-        // not depend on each other.
-        constexpr int NP = NT > 1 ? 2 : 1;
-#pragma unroll
-        for (int n = 0; n < NT; n += NP) {
-          double wd[NP][8];
-#pragma unroll
-          for (int p = 0; p < NP; p++) widen8(wq[d][n + p], wd[p]);
-#pragma unroll
-          for (int s = 0; s < 8; s++)
-#pragma unroll
-            for (int p = 0; p < NP; p++)
-              acc[n + p] = __builtin_amdgcn_mfma_f64_16x16x4f64(xd[s], wd[p][s], acc[n + p], 0, 0, 0);
-        }
-        load(d, c + D * WPC);
-      }
-    }
-  }
-
-#pragma unroll
-  for (int n = 0; n < NT; n++) {
-#pragma unroll
-    for (int i = 0; i < 4; i++) part[w][n][i][lane] = acc[n][i];
-  }
-  __syncthreads();
-
-  if (SPLIT) {
-    const int S = gridDim.y;
-    double *mine = ws + ((size_t)blockIdx.x * S + blockIdx.y) * (NT * 256);
-    for (int idx = tid; idx < NT * 4 * 64; idx += WPC * 64) {
-      double s = 0.0;
-#pragma unroll
-      for (int ww = 0; ww < WPC; ww++) s += (&part[ww][0][0][0])[idx];
-      mine[idx] = s;
-    }
-    __threadfence();  // the sums are out before the arrival is counted
-    __syncthreads();
-    if (tid == 0) is_last = atomicAdd(&arrivals[blockIdx.x], 1) == S - 1;
-    __syncthreads();
-    if (!is_last) return;
-    __threadfence();  // and the other workgroups' sums are read after it
-  }
-
-  // Result register i of lane l is token 4*i + l/16, expert 16*n + l%16.
-  for (int idx = tid; idx < NT * 4 * 64; idx += WPC * 64) {
-    const int l = idx & 63;
-    const int i = (idx >> 6) & 3;
-    const int n = idx >> 8;
-    double s = 0.0;
-    if (SPLIT) {
-      // all loads first (they are independent), then the sum in chunk order
-      const int S = gridDim.y;
-      const double *all = ws + (size_t)blockIdx.x * S * (NT * 256) + idx;
-      double v[kRouterSplitMax];
-#pragma unroll
-      for (int sp = 0; sp < kRouterSplitMax; sp++) v[sp] = sp < S ? all[(size_t)sp * (NT * 256)] : 0.0;
-#pragma unroll
-      for (int sp = 0; sp < kRouterSplitMax; sp++) s += v[sp];
-    } else {
-#pragma unroll
-      for (int ww = 0; ww < WPC; ww++) s += part[ww][n][i][l];
-    }
-    const int e = 16 * n + (l & 15);
-    const int tr = 4 * i + (l >> 4);
-    float f = (float)s;  // run.cpp:368
-    f += br[e];          // run.cpp:669-671
-    logits[tr][e] = f;
-    const int t = tok0 + tr;
-    if (score && e < E && t < T && !(pos && pos[t] < 0)) score[(size_t)t * E + e] = f;
-  }
-  __syncthreads();
-  if (SPLIT && tid == 0) arrivals[blockIdx.x] = 0;  // for the next launch
-
-  if (w != 0) return;
-  // Wave 0: four lanes per token, each owning a contiguous quarter of the experts.
-  constexpr int PER = E_pad / 4;
-  const int tr = lane >> 2;
-  const int q = lane & 3;
-  float v[PER];
-#pragma unroll
-  for (int j = 0; j < PER; j++) v[j] = logits[tr][q * PER + j];
-
-  float sel_v[kTopK];
-  int sel_i[kTopK];
-#pragma unroll
-  for (int r = 0; r < kTopK; r++) {
-    float best = -INFINITY;
-    int bi = 0x7fffffff;
+  for (int r = 0; r < NSEL; r++) {
+    float best = 0.f;
+    int bi = kNone;
 #pragma unroll
     for (int j = 0; j < PER; j++) {
-      if (v[j] > best) { best = v[j]; bi = q * PER + j; }
+      const int e = q * PER + j;
+      const bool ok = e < E && !((taken >> j) & 1ull);
+      if (ok && (bi == kNone || v[j] > best)) { best = v[j]; bi = e; }
     }
 #pragma unroll
     for (int off = 1; off < 4; off <<= 1) {
       const float ov = __shfl_xor(best, off, 64);
       const int oi = __shfl_xor(bi, off, 64);
-      if (ov > best || (ov == best && oi < bi)) { best = ov; bi = oi; }
+      // the lower index is the incumbent; kNone is above every index
+      const bool take = oi < bi ? !(bi != kNone && best > ov) : (oi != kNone && oi != bi && ov > best);
+      if (take) { best = ov; bi = oi; }
     }
     sel_v[r] = best;
     sel_i[r] = bi;
-#pragma unroll
-    for (int j = 0; j < PER; j++) {
-      if (q * PER + j == bi) v[j] = -INFINITY;
-    }
+    if (bi != kNone && bi / PER == q) taken |= 1ull << (bi % PER);
   }
-
-  const int t = tok0 + tr;
-  if (q != 0 || t >= T) return;
-  int4 oi;
-  float4 ov;
-  if (pos && pos[t] < 0) {
-    oi = make_int4(-1, -1, -1, -1);
-    ov = make_float4(0.f, 0.f, 0.f, 0.f);
-  } else {
-    // run.cpp:336-354 with size = 4; sel_v[0] is the maximum.
-    const double mx = (double)sel_v[0];
-    float ev[kTopK];
-    double sum = 0.0;
-#pragma unroll
-    for (int r = 0; r < kTopK; r++) {
-      ev[r] = expf((float)((double)sel_v[r] - mx));
-      sum += (double)ev[r];
-    }
-    oi = make_int4(sel_i[0], sel_i[1], sel_i[2], sel_i[3]);
-    ov = make_float4((float)((double)ev[0] / sum), (float)((double)ev[1] / sum),
-                     (float)((double)ev[2] / sum), (float)((double)ev[3] / sum));
-  }
-  *reinterpret_cast<int4 *>(topk_i + (size_t)t * kTopK) = oi;
-  *reinterpret_cast<float4 *>(topk_v + (size_t)t * kTopK) = ov;
 }
 
-// Chunks of 32 k per workgroup when a tile of 16 tokens is shared (0: no
-// sharing): batches of few tiles only, and never more than kRouterSplitMax
-// workgroups per tile.
-static int router_split_chunks(int T, int H) {
-  const int tiles = (T + 15) / 16;
+// run.cpp:336-354 with size = 4; v[0] is the maximum.
+__device__ __forceinline__ float4 softmax4(const float (&v)[kTopK]) {
+  const double mx = (double)v[0];
+  float ev[kTopK];
+  double sum = 0.0;
+#pragma unroll
+  for (int r = 0; r < kTopK; r++) {
+    ev[r] = expf((float)((double)v[r] - mx));
+    sum += (double)ev[r];
+  }
+  return make_float4((float)((double)ev[0] / sum), (float)((double)ev[1] / sum),
+                     (float)((double)ev[2] / sum), (float)((double)ev[3] / sum));
+}
+
+__device__ __forceinline__ void unpack8(const uint4 v, float (&f)[8]) {
+  f[0] = __uint_as_float(v.x << 16); f[1] = __uint_as_float(v.x & 0xffff0000u);
+  f[2] = __uint_as_float(v.y << 16); f[3] = __uint_as_float(v.y & 0xffff0000u);
+  f[4] = __uint_as_float(v.z << 16); f[5] = __uint_as_float(v.z & 0xffff0000u);
+  f[6] = __uint_as_float(v.w << 16); f[7] = __uint_as_float(v.w & 0xffff0000u);
+}
+
+// One workgroup = MT * 16 tokens x all experts (NT = E_pad / 16 blocks of 16).
+// Its WPC waves split the reduction dimension in chunks of 32 (wave w takes
+// chunks w, w + WPC, ...); D register sets of loads run ahead of the MFMAs.
+// rstat[0] = max_e |w_e| (slightly inflated), rstat[1] = max_e |b_e|.
+template <int NT, int WPC, int MT, int D>
+__global__ __launch_bounds__(WPC * 64) void router_kernel(
+    const uint16_t *__restrict__ x, const int *__restrict__ pos, const uint16_t *__restrict__ wr,
+    const float *__restrict__ br, const float *__restrict__ rstat, int T, int H, int E,
+    float *__restrict__ score, int *__restrict__ topk_i, float *__restrict__ topk_v) {
+  constexpr int E_pad = NT * 16;
+  constexpr int TOK = MT * 16;
+  static_assert(WPC >= MT, "one wave per 16 tokens does the selection");
+  __shared__ double sum64[MT][NT][4][64];  // [token tile][expert block][reg][lane]
+  __shared__ float sumsq[WPC][TOK];
+  __shared__ float logits[TOK][E_pad + 1];
+  __shared__ unsigned short tasks[TOK * E_pad];  // (token in tile) * E_pad + expert
+  __shared__ int n_tasks;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int w = tid >> 6;
+  const int tok0 = blockIdx.x * TOK;
+  const int row = lane & 15;  // token within a tile of 16 (first operand's row)
+  const int g = lane >> 4;    // which 8 of the chunk's 32 k this lane holds
   const int kc_total = H / 32;
-  if (tiles > kRouterSplitTiles) return 0;
-  const int cps = (kc_total + kRouterSplitMax - 1) / kRouterSplitMax;
-  return cps >= kc_total ? 0 : cps;
+  if (tid == 0) n_tasks = 0;
+
+  f32x4 acc32[MT][NT], nrm[MT];
+  double acc64[MT][NT][4];
+#pragma unroll
+  for (int m = 0; m < MT; m++) {
+    nrm[m] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int n = 0; n < NT; n++) {
+      acc32[m][n] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int i = 0; i < 4; i++) acc64[m][n][i] = 0.0;
+    }
+  }
+  auto flush = [&]() {
+#pragma unroll
+    for (int m = 0; m < MT; m++)
+#pragma unroll
+      for (int n = 0; n < NT; n++) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) acc64[m][n][i] += (double)acc32[m][n][i];
+        acc32[m][n] = f32x4{0.f, 0.f, 0.f, 0.f};
+      }
+  };
+
+  const uint16_t *xrow[MT];
+#pragma unroll
+  for (int m = 0; m < MT; m++) xrow[m] = x + (size_t)min(tok0 + 16 * m + row, T - 1) * H + g * 8;
+  const uint16_t *wlane = wr + (size_t)lane * 8;
+  uint4 xs[D][MT], wq[D][NT];
+  auto load = [&](int d, int c) {
+    const int cc = min(c, kc_total - 1);  // past the end the ring re-loads the last chunk and drops it
+#pragma unroll
+    for (int m = 0; m < MT; m++) xs[d][m] = *reinterpret_cast<const uint4 *>(xrow[m] + cc * 32);
+#pragma unroll
+    for (int n = 0; n < NT; n++)
+      wq[d][n] = *reinterpret_cast<const uint4 *>(wlane + ((size_t)n * kc_total + cc) * 512);
+  };
+#pragma unroll
+  for (int d = 0; d < D; d++) load(d, w + d * WPC);
+  int since_flush = 0;
+  for (int c0 = w; c0 < kc_total; c0 += D * WPC) {
+#pragma unroll
+    for (int d = 0; d < D; d++) {
+      const int c = c0 + d * WPC;
+      if (c < kc_total) {  // the same for the whole wave
+#pragma unroll
+        for (int m = 0; m < MT; m++) {
+          const bf16x8 xa = __builtin_bit_cast(bf16x8, xs[d][m]);
+#pragma unroll
+          for (int n = 0; n < NT; n++)
+            acc32[m][n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                xa, __builtin_bit_cast(bf16x8, wq[d][n]), acc32[m][n], 0, 0, 0);
+          nrm[m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xa, xa, nrm[m], 0, 0, 0);
+        }
+        load(d, c + D * WPC);
+        if (++since_flush == kFlush) {
+          flush();
+          since_flush = 0;
+        }
+      }
+    }
+  }
+  flush();
+
+  // |x_t|^2 is the diagonal of x x^T: register i of lane l is (row 4*(l/16) + i,
+  // column l % 16).
+  if ((row >> 2) == g) {
+#pragma unroll
+    for (int m = 0; m < MT; m++) {
+      const int i = row & 3;
+      sumsq[w][16 * m + row] = i == 0 ? nrm[m][0] : (i == 1 ? nrm[m][1] : (i == 2 ? nrm[m][2] : nrm[m][3]));
+    }
+  }
+  // The waves' fp64 sums are added up in wave order (the same sum in every run).
+  for (int ww = 0; ww < WPC; ww++) {
+    if (w == ww) {
+#pragma unroll
+      for (int m = 0; m < MT; m++)
+#pragma unroll
+        for (int n = 0; n < NT; n++)
+#pragma unroll
+          for (int i = 0; i < 4; i++) {
+            if (ww == 0) sum64[m][n][i][lane] = acc64[m][n][i];
+            else sum64[m][n][i][lane] += acc64[m][n][i];
+          }
+    }
+    __syncthreads();
+  }
+  // Register i of lane l is token 4*(l/16) + i of its tile, expert 16*n + l%16.
+  for (int idx = tid; idx < MT * NT * 256; idx += WPC * 64) {
+    const int l = idx & 63;
+    const int i = (idx >> 6) & 3;
+    const int n = (idx >> 8) % NT;
+    const int m = idx / (NT * 256);
+    const int e = 16 * n + (l & 15);
+    float f = (float)sum64[m][n][i][l];  // run.cpp:368
+    f += br[e];                          // run.cpp:669-671
+    logits[16 * m + 4 * (l >> 4) + i][e] = f;
+  }
+  __syncthreads();
+
+  // Pass 2, selection: wave m takes tile m, four lanes per token.
+  constexpr int PER = E_pad / 4;
+  const int tr = 16 * w + (lane >> 2);  // token within the workgroup (waves < MT only)
+  const int q = lane & 3;
+  const int t = tok0 + tr;
+  bool undecided = false;
+  if (w < MT) {
+    float v[PER];
+#pragma unroll
+    for (int j = 0; j < PER; j++) v[j] = logits[tr][q * PER + j];
+    float s_v[kTopK + 1];
+    int s_i[kTopK + 1];
+    select_top<PER, kTopK + 1>(v, q, E, s_v, s_i);
+    const bool active = t < T && !(pos && pos[t] < 0);
+    if (active) {
+      float ss = 0.f;
+#pragma unroll
+      for (int ww = 0; ww < WPC; ww++) ss += sumsq[ww][tr];
+      // bound on |first-pass logit - exact logit|: the accumulation error plus
+      // the two float roundings (sum -> float, + bias) of either arithmetic
+      const float err0 = kGamma * sqrtf(ss * 1.002f) * rstat[0];
+      const float bmax = rstat[1];
+      auto up = [&](float a) { return a + (4.76837158e-7f * (fabsf(a) + bmax) + err0); };
+      auto lo = [&](float a) { return a - (4.76837158e-7f * (fabsf(a) + bmax) + err0); };
+      const bool decided = lo(s_v[0]) > up(s_v[1]) && lo(s_v[1]) > up(s_v[2]) && lo(s_v[2]) > up(s_v[3]) &&
+                           (s_i[4] == kNone || lo(s_v[3]) > up(s_v[4]));
+      if (decided) {
+        if (q == 0) {
+          const float sv[kTopK] = {s_v[0], s_v[1], s_v[2], s_v[3]};
+          *reinterpret_cast<int4 *>(topk_i + (size_t)t * kTopK) = make_int4(s_i[0], s_i[1], s_i[2], s_i[3]);
+          *reinterpret_cast<float4 *>(topk_v + (size_t)t * kTopK) = softmax4(sv);
+        }
+      } else {
+        undecided = true;
+        // contenders: everything not provably below the fourth best (a NaN
+        // anywhere makes the comparison fail, and the expert a contender)
+        const float floor4 = lo(s_v[3]);
+#pragma unroll
+        for (int j = 0; j < PER; j++) {
+          const int e = q * PER + j;
+          if (e < E && !(up(v[j]) < floor4)) tasks[atomicAdd(&n_tasks, 1)] = (unsigned short)(tr * E_pad + e);
+        }
+      }
+    } else if (t < T && q == 0) {
+      *reinterpret_cast<int4 *>(topk_i + (size_t)t * kTopK) = make_int4(-1, -1, -1, -1);
+      *reinterpret_cast<float4 *>(topk_v + (size_t)t * kTopK) = make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+  }
+  __syncthreads();
+
+  // Exact logits of the contenders, one wave per (token, expert): float
+  // products, fp64 sum, one rounding to float, bias added in float.
+  const int nt = n_tasks;
+  for (int task = w; task < nt; task += WPC) {
+    const int code = tasks[task];
+    const int tt = code / E_pad, e = code % E_pad;
+    const uint16_t *xr = x + (size_t)min(tok0 + tt, T - 1) * H;
+    const uint16_t *we = wr + ((size_t)(e >> 4) * kc_total * 64 + (e & 15)) * 8;
+    double s = 0.0;
+    for (int p = lane; p < H / 8; p += 64) {  // piece p: k = 8p .. 8p+7 = chunk p/4, quarter p%4
+      const uint4 xv = *reinterpret_cast<const uint4 *>(xr + p * 8);
+      const uint4 wv = *reinterpret_cast<const uint4 *>(we + ((size_t)(p >> 2) * 64 + (p & 3) * 16) * 8);
+      float xf[8], wf[8];
+      unpack8(xv, xf);
+      unpack8(wv, wf);
+#pragma unroll
+      for (int j = 0; j < 8; j++) s += (double)(xf[j] * wf[j]);
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) s += __shfl_xor(s, off, 64);
+    if (lane == 0) {
+      float f = (float)s;
+      f += br[e];
+      logits[tt][e] = f;
+    }
+  }
+  __syncthreads();
+
+  if (undecided) {  // waves < MT only
+    float v[PER];
+#pragma unroll
+    for (int j = 0; j < PER; j++) v[j] = logits[tr][q * PER + j];
+    float s_v[kTopK];
+    int s_i[kTopK];
+    select_top<PER, kTopK>(v, q, E, s_v, s_i);
+    if (q == 0) {
+      *reinterpret_cast<int4 *>(topk_i + (size_t)t * kTopK) = make_int4(s_i[0], s_i[1], s_i[2], s_i[3]);
+      *reinterpret_cast<float4 *>(topk_v + (size_t)t * kTopK) = softmax4(s_v);
+    }
+  }
+  if (score) {
+    for (int idx = tid; idx < TOK * E_pad; idx += WPC * 64) {
+      const int tt = idx / E_pad, e = idx % E_pad;
+      const int ts = tok0 + tt;
+      if (e < E && ts < T && !(pos && pos[ts] < 0)) score[(size_t)ts * E + e] = logits[tt][e];
+    }
+  }
+}
+
+// Statistics of a layer's router for the error bound of the first pass:
+// rstat[0] = max_e |w_e|_2 over the bf16-rounded weights (inflated by 1e-3 for
+// the rounding of this very sum), rstat[1] = max_e |b_e|.  One workgroup.
+__global__ __launch_bounds__(256) void router_stats_kernel(const float *__restrict__ w,
+                                                           const float *__restrict__ b, int E, int H,
+                                                           float *__restrict__ rstat) {
+  __shared__ float red[256];
+  float wmax = 0.f, bmax = 0.f;
+  for (int e = 0; e < E; e++) {
+    float s = 0.f;
+    for (int k = threadIdx.x; k < H; k += 256) {
+      const float v = __uint_as_float((uint32_t)f32_to_bf16_rne(w[(size_t)e * H + k]) << 16);
+      s += v * v;
+    }
+    red[threadIdx.x] = s;
+    __syncthreads();
+    for (int off = 128; off > 0; off >>= 1) {
+      if ((int)threadIdx.x < off) red[threadIdx.x] += red[threadIdx.x + off];
+      __syncthreads();
+    }
+    wmax = fmaxf(wmax, red[0]);
+    __syncthreads();
+    bmax = fmaxf(bmax, fabsf(__uint_as_float((uint32_t)f32_to_bf16_rne(b[e]) << 16)));
+  }
+  if (threadIdx.x == 0) {
+    rstat[0] = sqrtf(wmax) * 1.001f;
+    rstat[1] = bmax;
+  }
+}
+
+hipError_t launch_router_stats(const float *w_src, const float *b_src, int E, int H, float *rstat,
+                               hipStream_t s) {
+  router_stats_kernel<<<1, 256, 0, s>>>(w_src, b_src, E, H, rstat);
+  return hipGetLastError();
 }
 
 template <int NT>
 static hipError_t launch_router_nt(const uint16_t *x, const int *pos, const uint16_t *wr,
-                                   const float *br, int T, int H, int E, float *score, int *topk_i,
-                                   float *topk_v, double *ws, int *arrivals, hipStream_t s) {
-  const int grid = (T + 15) / 16;
-  // Register sets in flight per wave, 4 * (1 + NT) registers each, within the
-  // 128 / 256 / 512 registers a wave of a workgroup this size can have.
+                                   const float *br, const float *rstat, int T, int H, int E,
+                                   float *score, int *topk_i, float *topk_v, hipStream_t s) {
+  // As fine a split of the reduction as the registers allow: more waves keep
+  // more loads in flight, and small batches still occupy the SIMDs.  D register
+  // sets of 4 * (MT + NT) registers each run ahead.
+  constexpr int WPC = NT <= 2 ? 16 : (NT <= 4 ? 8 : 4);
   constexpr int D = NT <= 2 ? 6 : (NT <= 4 ? 4 : (NT <= 8 ? 3 : 2));
-  const int cps = ws ? router_split_chunks(T, H) : 0;
-  if (cps > 0) {
-    constexpr int WPS = NT <= 8 ? 4 : 2;  // waves of a workgroup that shares a tile
-    constexpr int DS = D < 3 ? D : 3;
-    const int S = (H / 32 + cps - 1) / cps;
-    router_kernel<NT, WPS, DS, true><<<dim3(grid, S), WPS * 64, 0, s>>>(x, pos, wr, br, T, H, E, score, topk_i,
-                                                                        topk_v, ws, arrivals, cps);
-    return hipGetLastError();
+  // Every workgroup streams the whole router matrix through its CU; at 128
+  // experts a workgroup takes two tiles of 16 tokens so that half as many do
+  // (at 256 the accumulators of two tiles no longer fit the registers).
+  if (NT == 8 && T > 256 * 16) {
+    constexpr int MT = NT == 8 ? 2 : 1;
+    router_kernel<NT, WPC, MT, D><<<(T + 16 * MT - 1) / (16 * MT), WPC * 64, 0, s>>>(
+        x, pos, wr, br, rstat, T, H, E, score, topk_i, topk_v);
+  } else {
+    router_kernel<NT, WPC, 1, D><<<(T + 15) / 16, WPC * 64, 0, s>>>(x, pos, wr, br, rstat, T, H, E, score,
+                                                                   topk_i, topk_v);
   }
-  // As many waves per workgroup (i.e. as fine a split of the reduction) as the
-  // LDS for the partial sums allows (WPC * NT * 2 KB <= 64 KB): more waves per
-  // SIMD hide the load latency, and small batches still occupy the SIMDs.
-  constexpr int WPC = NT <= 2 ? 16 : (NT <= 4 ? 8 : (NT <= 8 ? 4 : 2));
-  router_kernel<NT, WPC, D, false><<<grid, WPC * 64, 0, s>>>(x, pos, wr, br, T, H, E, score, topk_i,
-                                                             topk_v, nullptr, nullptr, 0);
   return hipGetLastError();
 }
 
-hipError_t launch_router(const uint16_t *x, const int *pos, const uint16_t *wr, const float *br, int T,
-                         int H, int E, int E_pad, float *score, int *topk_i, float *topk_v,
-                         double *ws, int *arrivals, hipStream_t s) {
+hipError_t launch_router(const uint16_t *x, const int *pos, const uint16_t *wr, const float *br,
+                         const float *rstat, int T, int H, int E, int E_pad, float *score, int *topk_i,
+                         float *topk_v, hipStream_t s) {
   if (T <= 0) return hipSuccess;
   switch (E_pad / 16) {
-    case 1: return launch_router_nt<1>(x, pos, wr, br, T, H, E, score, topk_i, topk_v, ws, arrivals, s);
-    case 2: return launch_router_nt<2>(x, pos, wr, br, T, H, E, score, topk_i, topk_v, ws, arrivals, s);
-    case 4: return launch_router_nt<4>(x, pos, wr, br, T, H, E, score, topk_i, topk_v, ws, arrivals, s);
-    case 8: return launch_router_nt<8>(x, pos, wr, br, T, H, E, score, topk_i, topk_v, ws, arrivals, s);
-    case 16: return launch_router_nt<16>(x, pos, wr, br, T, H, E, score, topk_i, topk_v, ws, arrivals, s);
+    case 1: return launch_router_nt<1>(x, pos, wr, br, rstat, T, H, E, score, topk_i, topk_v, s);
+    case 2: return launch_router_nt<2>(x, pos, wr, br, rstat, T, H, E, score, topk_i, topk_v, s);
+    case 4: return launch_router_nt<4>(x, pos, wr, br, rstat, T, H, E, score, topk_i, topk_v, s);
+    case 8: return launch_router_nt<8>(x, pos, wr, br, rstat, T, H, E, score, topk_i, topk_v, s);
+    case 16: return launch_router_nt<16>(x, pos, wr, br, rstat, T, H, E, score, topk_i, topk_v, s);
     default: return hipErrorInvalidValue;
   }
 }

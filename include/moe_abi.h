@@ -167,6 +167,23 @@ int moe_experts(moe_handle *h, int layer, const uint16_t *x, const int *pos,
                 const int *topk_i, const float *topk_v, int n_tokens,
                 float *out, int accumulate, void *stream);
 
+/* Stages 3-5 alone, on the plan of the last moe_dispatch of the same batch:
+ * gathers the routed rows of x into per-expert segments, runs the gate_up
+ * grouped GEMM with the clamped SwiGLU and the down grouped GEMM, and leaves one
+ * fp32 row per assignment inside the handle.  Replaces the mlp1 / mlp2 launches
+ * of the local path (getp_run.cpp:788-829; kernels matmul/matmul.cpp:1023-1914). */
+int moe_expert_gemms(moe_handle *h, int layer, const uint16_t *x, int n_tokens,
+                     void *stream);
+
+/* Stage 6 alone, after moe_dispatch and moe_expert_gemms of the same batch:
+ * out[t,:] (+)= sum_k topk_v[t,k] * (row of assignment t*K+k), slots added in
+ * order 0..K-1, rows with pos < 0 skipped (accumulate) or zeroed.  Replaces
+ * reduce_mlp2_slots_kernel (utility/utility.cpp:701-726, launched at
+ * getp_run.cpp:831-843); the routing weight is applied here, in fp32, rather
+ * than in the down GEMM's epilogue (matmul/matmul.cpp:1868-1870). */
+int moe_combine(moe_handle *h, const float *topk_v, const int *pos, int n_tokens,
+                float *out, int accumulate, void *stream);
+
 /* Per-stage timing with HIP events on the stream of the forward calls.
  * moe_profile_enable(h, n) arms timing for the next n forward calls (n <= 256);
  * moe_profile_read synchronises on the recorded events and returns the mean

@@ -51,6 +51,31 @@ def check_routing(R, L, x, pos, E):
     return ti, off
 
 
+def stratified_rows(R, E, cap=640, seed=0):
+    """Token rows that cover the GEMMs' tile plan: for every expert one row out
+    of each of its row blocks of 32 (always from the first and the last block, so
+    every row-block position of every tile height is hit, the ragged last block
+    included), at varying places inside the block, thinned evenly down to about
+    `cap` tokens."""
+    off, perm = R["offsets"], R["perm"]
+    must, rest = [], []
+    for e in range(E):
+        n = int(off[e + 1] - off[e])
+        n_blk = (n + 31) // 32
+        for b in range(n_blk):
+            r = min(32 * b + (7 * b + e) % 32, n - 1)
+            tok = int(perm[off[e] + r]) // 4
+            (must if b in (0, n_blk - 1) else rest).append(tok)
+        if n:
+            must.append(int(perm[off[e] + n - 1]) // 4)  # the segment's very last row
+    must = sorted(set(must))
+    rest = sorted(set(rest) - set(must))
+    room = max(cap - len(must), 0)
+    if len(rest) > room:
+        rest = list(np.random.default_rng(seed).choice(rest, room, replace=False))
+    return np.array(sorted(set(must) | set(int(t) for t in rest)), dtype=np.int64)
+
+
 def check_outputs(R, L, x, pos, rows, limit=7.0):
     want = oracle_rows(L, x, pos, rows, limit)
     got = R["out"][rows]
@@ -170,9 +195,10 @@ def test_c2_full_batch(c2):
     _, off = check_routing(R, L, L["x"], None, sh.experts)
     counts = np.diff(off)
     assert counts.sum() == 4 * T and counts.min() > 300  # roughly uniform load
-    rows = np.random.default_rng(0).choice(T, 48, replace=False)
-    err = check_outputs(R, L, L["x"], None, np.sort(rows))
-    print(f"c2 rel-L2 vs oracle on 48 rows: {err:.2e}; rows per expert {counts.min()}..{counts.max()}")
+    rows = stratified_rows(R, sh.experts)
+    assert len(rows) >= 512
+    err = check_outputs(R, L, L["x"], None, rows)
+    print(f"c2 rel-L2 vs oracle on {len(rows)} rows: {err:.2e}; rows per expert {counts.min()}..{counts.max()}")
     assert np.isfinite(R["out"]).all()
 
 
@@ -237,7 +263,8 @@ def test_c3_zipf_routing(name, c2):
         counts = np.diff(off)
         print(f"{name}: rows per expert max {counts.max()} min {counts.min()} (T={sh.tokens})")
         assert counts.max() > 6 * max(counts.min(), 1)  # the load really is skewed
-        rows = np.sort(np.random.default_rng(4).choice(sh.tokens, 32, replace=False))
+        rows = stratified_rows(R, sh.experts, cap=640 if name == "c3b" else 200)
+        assert len(rows) >= (512 if name == "c3b" else 64)
         check_outputs(R, L, x, None, rows)
     finally:
         m.upload_layer(0, *[L2[k] for k in W])
@@ -299,8 +326,18 @@ def test_c4_120b_shape():
     m = make_moe(sh, L, sh.tokens)
     R = abi.run_layer(m, 0, L["x"], None)
     check_routing(R, L, L["x"], None, sh.experts)
-    rows = np.sort(np.random.default_rng(5).choice(sh.tokens, 32, replace=False))
+    rows = stratified_rows(R, sh.experts)
+    assert len(rows) >= 512
     check_outputs(R, L, L["x"], None, rows)
+    # the large-batch GEMMs at 128 experts, twelve calls: same bits every time
+    T = sh.tokens
+    dx = abi.DevBuf.from_numpy(synth.to_bf16_bits(L["x"]))
+    dout = abi.DevBuf(T * sh.hidden * 4)
+    for i in range(12):
+        dout.memset(0xFF)
+        m.forward(0, dx, None, T, dout)
+        abi.sync()
+        assert np.array_equal(dout.download((T, sh.hidden), np.float32), R["out"]), f"call {i} gave other bits"
 
 
 def test_c5_mxfp4_ingest():
