@@ -9,9 +9,10 @@
 // Two passes in one kernel:
 //   1. All logits on the bf16 matrix cores (v_mfma_f32_16x16x32_bf16).  The
 //      products are exact; the fp32 accumulation inside the matrix core is not,
-//      so a wave hands its fp32 sums over to fp64 accumulators every kFlush
-//      MFMAs.  That bounds the error of a logit by kGamma * sum_k |x_k w_ek|
-//      <= kGamma * |x| * |w_e| (Cauchy-Schwarz; |x|^2 comes out of one more
+//      so a wave hands its fp32 sums over to fp64 accumulators every FLUSH
+//      MFMAs (every one while the experts are few and the hand-over is cheap).
+//      That bounds the error of a logit by gamma * sum_k |x_k w_ek|
+//      <= gamma * |x| * |w_e| (Cauchy-Schwarz; |x|^2 comes out of one more
 //      MFMA per chunk, x times its own transpose, and max_e |w_e| is computed
 //      at upload).
 //   2. A token whose five best logits are further apart than twice that bound
@@ -35,24 +36,24 @@ namespace moe {
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
-constexpr int kFlush = 4;  // MFMAs (of 32 k) between two hand-overs to fp64
-// Error of one fp32 chain of kFlush MFMAs started from zero, relative to the
-// sum of the magnitudes of its 32 * kFlush products: every one of its
-// 33 * kFlush additions is taken to lose at most 2^-23 of the running
+// Error of one fp32 chain of `flush` MFMAs (of 32 k each) started from zero,
+// relative to the sum of the magnitudes of its 32 * flush products: every one
+// of its 33 * flush additions is taken to lose at most 2^-23 of the running
 // magnitude (covers truncation as well as rounding), and the result is doubled.
-constexpr float kGamma = 2.0f * 33.0f * kFlush * 1.1920929e-7f;
+__host__ __device__ constexpr float router_gamma(int flush) { return 2.0f * 33.0f * flush * 1.1920929e-7f; }
 constexpr int kNone = 0x7fffffff;
 
-// Top-NSEL of a token's logits held by four lanes (lane q owns experts
-// q*PER .. q*PER+PER-1), by the rule of the reference's CPU top-k under a stable
+// Top-NSEL of a token's logits held by LPT neighbouring lanes (lane q of them
+// owns experts q*PER .. q*PER+PER-1), by the rule of the reference's CPU top-k under a stable
 // sort: value descending, index ascending; a candidate replaces the incumbent
 // (the one with the lower index) only if it compares strictly greater, so a
 // NaN neither wins nor loses a comparison and a row of NaNs selects 0, 1, 2, 3.
-// Experts >= E are never selected.  All four lanes end with the same result.
-template <int PER, int NSEL>
+// Experts >= E are never selected.  All LPT lanes end with the same result.
+template <int PER, int LPT, int NSEL>
 __device__ __forceinline__ void select_top(const float (&v)[PER], int q, int E, float (&sel_v)[NSEL],
                                            int (&sel_i)[NSEL]) {
-  unsigned long long taken = 0;
+  static_assert(PER <= 32, "one bit per owned expert");
+  unsigned taken = 0;
 #pragma unroll
   for (int r = 0; r < NSEL; r++) {
     float best = 0.f;
@@ -60,11 +61,11 @@ __device__ __forceinline__ void select_top(const float (&v)[PER], int q, int E, 
 #pragma unroll
     for (int j = 0; j < PER; j++) {
       const int e = q * PER + j;
-      const bool ok = e < E && !((taken >> j) & 1ull);
+      const bool ok = e < E && !((taken >> j) & 1u);
       if (ok && (bi == kNone || v[j] > best)) { best = v[j]; bi = e; }
     }
 #pragma unroll
-    for (int off = 1; off < 4; off <<= 1) {
+    for (int off = 1; off < LPT; off <<= 1) {
       const float ov = __shfl_xor(best, off, 64);
       const int oi = __shfl_xor(bi, off, 64);
       // the lower index is the incumbent; kNone is above every index
@@ -73,7 +74,7 @@ __device__ __forceinline__ void select_top(const float (&v)[PER], int q, int E, 
     }
     sel_v[r] = best;
     sel_i[r] = bi;
-    if (bi != kNone && bi / PER == q) taken |= 1ull << (bi % PER);
+    if (bi != kNone && bi / PER == q) taken |= 1u << (bi % PER);
   }
 }
 
@@ -102,19 +103,28 @@ __device__ __forceinline__ void unpack8(const uint4 v, float (&f)[8]) {
 // Its WPC waves split the reduction dimension in chunks of 32 (wave w takes
 // chunks w, w + WPC, ...); D register sets of loads run ahead of the MFMAs.
 // rstat[0] = max_e |w_e| (slightly inflated), rstat[1] = max_e |b_e|.
-template <int NT, int WPC, int MT, int D>
+template <int NT, int WPC, int MT, int D, int FLUSH>
 __global__ __launch_bounds__(WPC * 64) void router_kernel(
     const uint16_t *__restrict__ x, const int *__restrict__ pos, const uint16_t *__restrict__ wr,
     const float *__restrict__ br, const float *__restrict__ rstat, int T, int H, int E,
     float *__restrict__ score, int *__restrict__ topk_i, float *__restrict__ topk_v) {
   constexpr int E_pad = NT * 16;
   constexpr int TOK = MT * 16;
-  static_assert(WPC >= MT, "one wave per 16 tokens does the selection");
-  __shared__ double sum64[MT][NT][4][64];  // [token tile][expert block][reg][lane]
+  // selection: LPT lanes per token, each owning PER experts; SW waves take part
+  constexpr int LPT = E_pad <= 64 ? 4 : (E_pad == 128 ? 8 : 16);
+  constexpr int PER = E_pad / LPT;
+  constexpr int SW = TOK * LPT / 64;
+  static_assert(SW >= 1 && SW <= WPC, "waves of the selection");
+  // cross-wave sum: GB blocks of 16 x 16 outputs at a time through 32 KB
+  constexpr int NBLK = MT * NT;
+  constexpr int GB = 32 / WPC < NBLK ? 32 / WPC : NBLK;
+  static_assert(WPC >= 2 && NBLK % GB == 0, "groups of the cross-wave sum");
+  __shared__ double part[WPC / 2][GB][4][64];  // [wave][block][reg][lane]
   __shared__ float sumsq[WPC][TOK];
   __shared__ float logits[TOK][E_pad + 1];
   __shared__ unsigned short tasks[TOK * E_pad];  // (token in tile) * E_pad + expert
   __shared__ int n_tasks;
+  __shared__ float sh_br[E_pad];  // the bias, fetched while the first pass runs
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -124,6 +134,13 @@ __global__ __launch_bounds__(WPC * 64) void router_kernel(
   const int g = lane >> 4;    // which 8 of the chunk's 32 k this lane holds
   const int kc_total = H / 32;
   if (tid == 0) n_tasks = 0;
+  if (tid < E_pad) sh_br[tid] = br[tid];
+  // the selection's own inputs, loaded long before they are needed
+  const int tr = w * (64 / LPT) + lane / LPT;  // token within the workgroup (waves < SW only)
+  const int q = lane % LPT;
+  const int t = tok0 + tr;
+  const bool active = w < SW && t < T && !(pos && pos[min(t, T - 1)] < 0);
+  const float wn_max = rstat[0], bmax = rstat[1];
 
   f32x4 acc32[MT][NT], nrm[MT];
   double acc64[MT][NT][4];
@@ -154,7 +171,7 @@ __global__ __launch_bounds__(WPC * 64) void router_kernel(
   const uint16_t *wlane = wr + (size_t)lane * 8;
   uint4 xs[D][MT], wq[D][NT];
   auto load = [&](int d, int c) {
-    const int cc = min(c, kc_total - 1);  // past the end the ring re-loads the last chunk and drops it
+    const int cc = min(c, kc_total - 1);  // only the first D loads of a wave can lie past the end
 #pragma unroll
     for (int m = 0; m < MT; m++) xs[d][m] = *reinterpret_cast<const uint4 *>(xrow[m] + cc * 32);
 #pragma unroll
@@ -178,8 +195,8 @@ __global__ __launch_bounds__(WPC * 64) void router_kernel(
                 xa, __builtin_bit_cast(bf16x8, wq[d][n]), acc32[m][n], 0, 0, 0);
           nrm[m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xa, xa, nrm[m], 0, 0, 0);
         }
-        load(d, c + D * WPC);
-        if (++since_flush == kFlush) {
+        if (c + D * WPC < kc_total) load(d, c + D * WPC);  // nothing is loaded that is not used
+        if (FLUSH == 1 || ++since_flush == FLUSH) {
           flush();
           since_flush = 0;
         }
@@ -197,56 +214,59 @@ __global__ __launch_bounds__(WPC * 64) void router_kernel(
       sumsq[w][16 * m + row] = i == 0 ? nrm[m][0] : (i == 1 ? nrm[m][1] : (i == 2 ? nrm[m][2] : nrm[m][3]));
     }
   }
-  // The waves' fp64 sums are added up in wave order (the same sum in every run).
-  for (int ww = 0; ww < WPC; ww++) {
-    if (w == ww) {
+  // The waves' fp64 sums are added up in a fixed order (the same sum in every
+  // run): the upper half of the waves hands its sums to the lower half, whose
+  // results all threads then add in wave order; GB blocks at a time.
 #pragma unroll
-      for (int m = 0; m < MT; m++)
+  for (int b0 = 0; b0 < NBLK; b0 += GB) {
+    if (w >= WPC / 2) {
 #pragma unroll
-        for (int n = 0; n < NT; n++)
+      for (int b = 0; b < GB; b++)
 #pragma unroll
-          for (int i = 0; i < 4; i++) {
-            if (ww == 0) sum64[m][n][i][lane] = acc64[m][n][i];
-            else sum64[m][n][i][lane] += acc64[m][n][i];
-          }
+        for (int i = 0; i < 4; i++) part[w - WPC / 2][b][i][lane] = acc64[(b0 + b) / NT][(b0 + b) % NT][i];
+    }
+    __syncthreads();
+    if (w < WPC / 2) {
+#pragma unroll
+      for (int b = 0; b < GB; b++)
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+          part[w][b][i][lane] += acc64[(b0 + b) / NT][(b0 + b) % NT][i];
+    }
+    __syncthreads();
+    // Register i of lane l is token 4*(l/16) + i of its tile, expert 16*n + l%16.
+    for (int idx = tid; idx < GB * 256; idx += WPC * 64) {
+      const int l = idx & 63;
+      const int i = (idx >> 6) & 3;
+      const int b = b0 + (idx >> 8);
+      const int m = b / NT, n = b % NT;
+      const int e = 16 * n + (l & 15);
+      double sd = 0.0;
+#pragma unroll
+      for (int ww = 0; ww < WPC / 2; ww++) sd += part[ww][idx >> 8][i][l];
+      float f = (float)sd;  // run.cpp:368
+      f += sh_br[e];        // run.cpp:669-671
+      logits[16 * m + 4 * (l >> 4) + i][e] = f;
     }
     __syncthreads();
   }
-  // Register i of lane l is token 4*(l/16) + i of its tile, expert 16*n + l%16.
-  for (int idx = tid; idx < MT * NT * 256; idx += WPC * 64) {
-    const int l = idx & 63;
-    const int i = (idx >> 6) & 3;
-    const int n = (idx >> 8) % NT;
-    const int m = idx / (NT * 256);
-    const int e = 16 * n + (l & 15);
-    float f = (float)sum64[m][n][i][l];  // run.cpp:368
-    f += br[e];                          // run.cpp:669-671
-    logits[16 * m + 4 * (l >> 4) + i][e] = f;
-  }
-  __syncthreads();
 
-  // Pass 2, selection: wave m takes tile m, four lanes per token.
-  constexpr int PER = E_pad / 4;
-  const int tr = 16 * w + (lane >> 2);  // token within the workgroup (waves < MT only)
-  const int q = lane & 3;
-  const int t = tok0 + tr;
+  // Pass 2, selection: LPT lanes per token.
   bool undecided = false;
-  if (w < MT) {
+  if (w < SW) {
     float v[PER];
 #pragma unroll
     for (int j = 0; j < PER; j++) v[j] = logits[tr][q * PER + j];
     float s_v[kTopK + 1];
     int s_i[kTopK + 1];
-    select_top<PER, kTopK + 1>(v, q, E, s_v, s_i);
-    const bool active = t < T && !(pos && pos[t] < 0);
+    select_top<PER, LPT, kTopK + 1>(v, q, E, s_v, s_i);
     if (active) {
       float ss = 0.f;
 #pragma unroll
       for (int ww = 0; ww < WPC; ww++) ss += sumsq[ww][tr];
       // bound on |first-pass logit - exact logit|: the accumulation error plus
       // the two float roundings (sum -> float, + bias) of either arithmetic
-      const float err0 = kGamma * sqrtf(ss * 1.002f) * rstat[0];
-      const float bmax = rstat[1];
+      const float err0 = router_gamma(FLUSH) * sqrtf(ss * 1.002f) * wn_max;
       auto up = [&](float a) { return a + (4.76837158e-7f * (fabsf(a) + bmax) + err0); };
       auto lo = [&](float a) { return a - (4.76837158e-7f * (fabsf(a) + bmax) + err0); };
       const bool decided = lo(s_v[0]) > up(s_v[1]) && lo(s_v[1]) > up(s_v[2]) && lo(s_v[2]) > up(s_v[3]) &&
@@ -276,40 +296,71 @@ __global__ __launch_bounds__(WPC * 64) void router_kernel(
   __syncthreads();
 
   // Exact logits of the contenders, one wave per (token, expert): float
-  // products, fp64 sum, one rounding to float, bias added in float.
+  // products, fp64 sum, one rounding to float, bias added in float.  A wave
+  // takes TPW tasks at a time and has all their loads in flight at once (the
+  // phase is a chain of memory round trips otherwise).
+  constexpr int TPW = WPC >= 8 ? 1 : 2;
+  constexpr int PIECES = 6;  // 16-byte pieces per lane and operand in one round: 3072 k
   const int nt = n_tasks;
-  for (int task = w; task < nt; task += WPC) {
-    const int code = tasks[task];
-    const int tt = code / E_pad, e = code % E_pad;
-    const uint16_t *xr = x + (size_t)min(tok0 + tt, T - 1) * H;
-    const uint16_t *we = wr + ((size_t)(e >> 4) * kc_total * 64 + (e & 15)) * 8;
-    double s = 0.0;
-    for (int p = lane; p < H / 8; p += 64) {  // piece p: k = 8p .. 8p+7 = chunk p/4, quarter p%4
-      const uint4 xv = *reinterpret_cast<const uint4 *>(xr + p * 8);
-      const uint4 wv = *reinterpret_cast<const uint4 *>(we + ((size_t)(p >> 2) * 64 + (p & 3) * 16) * 8);
-      float xf[8], wf[8];
-      unpack8(xv, xf);
-      unpack8(wv, wf);
+  const int n_pieces = H / 8;
+  for (int task0 = w * TPW; task0 < nt; task0 += WPC * TPW) {
+    double s[TPW];
+    const uint16_t *xr[TPW], *we[TPW];
+    int tt[TPW], ee[TPW];
 #pragma unroll
-      for (int j = 0; j < 8; j++) s += (double)(xf[j] * wf[j]);
+    for (int j = 0; j < TPW; j++) {
+      const int code = tasks[min(task0 + j, nt - 1)];
+      tt[j] = code / E_pad;
+      ee[j] = code % E_pad;
+      xr[j] = x + (size_t)min(tok0 + tt[j], T - 1) * H;
+      we[j] = wr + ((size_t)(ee[j] >> 4) * kc_total * 64 + (ee[j] & 15)) * 8;
+      s[j] = 0.0;
+    }
+    for (int p0 = 0; p0 < n_pieces; p0 += 64 * PIECES) {
+      uint4 xv[TPW][PIECES], wv[TPW][PIECES];
+#pragma unroll
+      for (int j = 0; j < TPW; j++)
+#pragma unroll
+        for (int i = 0; i < PIECES; i++) {
+          // piece p: k = 8p .. 8p+7 = chunk p/4, quarter p%4; past the row's end: piece 0, not used
+          const int pp = p0 + i * 64 + lane;
+          const int p = pp < n_pieces ? pp : 0;
+          xv[j][i] = *reinterpret_cast<const uint4 *>(xr[j] + p * 8);
+          wv[j][i] = *reinterpret_cast<const uint4 *>(we[j] + ((size_t)(p >> 2) * 64 + (p & 3) * 16) * 8);
+        }
+#pragma unroll
+      for (int j = 0; j < TPW; j++)
+#pragma unroll
+        for (int i = 0; i < PIECES; i++) {
+          if (p0 + i * 64 + lane < n_pieces) {
+            float xf[8], wf[8];
+            unpack8(xv[j][i], xf);
+            unpack8(wv[j][i], wf);
+#pragma unroll
+            for (int k = 0; k < 8; k++) s[j] += (double)(xf[k] * wf[k]);
+          }
+        }
     }
 #pragma unroll
-    for (int off = 32; off > 0; off >>= 1) s += __shfl_xor(s, off, 64);
-    if (lane == 0) {
-      float f = (float)s;
-      f += br[e];
-      logits[tt][e] = f;
+    for (int j = 0; j < TPW; j++) {
+#pragma unroll
+      for (int off = 32; off > 0; off >>= 1) s[j] += __shfl_xor(s[j], off, 64);
+      if (lane == 0 && task0 + j < nt) {
+        float f = (float)s[j];
+        f += sh_br[ee[j]];
+        logits[tt[j]][ee[j]] = f;
+      }
     }
   }
   __syncthreads();
 
-  if (undecided) {  // waves < MT only
+  if (undecided) {  // waves < SW only
     float v[PER];
 #pragma unroll
     for (int j = 0; j < PER; j++) v[j] = logits[tr][q * PER + j];
     float s_v[kTopK];
     int s_i[kTopK];
-    select_top<PER, kTopK>(v, q, E, s_v, s_i);
+    select_top<PER, LPT, kTopK>(v, q, E, s_v, s_i);
     if (q == 0) {
       *reinterpret_cast<int4 *>(topk_i + (size_t)t * kTopK) = make_int4(s_i[0], s_i[1], s_i[2], s_i[3]);
       *reinterpret_cast<float4 *>(topk_v + (size_t)t * kTopK) = softmax4(s_v);
@@ -369,16 +420,21 @@ static hipError_t launch_router_nt(const uint16_t *x, const int *pos, const uint
   // sets of 4 * (MT + NT) registers each run ahead.
   constexpr int WPC = NT <= 2 ? 16 : (NT <= 4 ? 8 : 4);
   constexpr int D = NT <= 2 ? 6 : (NT <= 4 ? 4 : (NT <= 8 ? 3 : 2));
+  // MFMAs between two hand-overs to fp64: the fewer, the tighter the bound and
+  // the fewer tokens take the second pass, at 8 * NT more fp64 instructions
+  // each; the first pass is bound by its loads, so the hand-over after every
+  // MFMA costs nothing
+  constexpr int FLUSH = 1;
   // Every workgroup streams the whole router matrix through its CU; at 128
   // experts a workgroup takes two tiles of 16 tokens so that half as many do
   // (at 256 the accumulators of two tiles no longer fit the registers).
   if (NT == 8 && T > 256 * 16) {
     constexpr int MT = NT == 8 ? 2 : 1;
-    router_kernel<NT, WPC, MT, D><<<(T + 16 * MT - 1) / (16 * MT), WPC * 64, 0, s>>>(
+    router_kernel<NT, WPC, MT, D, FLUSH><<<(T + 16 * MT - 1) / (16 * MT), WPC * 64, 0, s>>>(
         x, pos, wr, br, rstat, T, H, E, score, topk_i, topk_v);
   } else {
-    router_kernel<NT, WPC, 1, D><<<(T + 15) / 16, WPC * 64, 0, s>>>(x, pos, wr, br, rstat, T, H, E, score,
-                                                                   topk_i, topk_v);
+    router_kernel<NT, WPC, 1, D, FLUSH><<<(T + 15) / 16, WPC * 64, 0, s>>>(x, pos, wr, br, rstat, T, H, E,
+                                                                          score, topk_i, topk_v);
   }
   return hipGetLastError();
 }

@@ -43,7 +43,9 @@ def check_routing(R, L, x, pos, E):
     off, perm, _ = ob.dispatch(ti, pos, E)
     assert np.array_equal(R["topk_i"], ti), "expert ids differ from the oracle"
     act = np.ones(x.shape[0], bool) if pos is None else pos >= 0
-    np.testing.assert_allclose(R["score"][act], score[act], rtol=0, atol=2e-6)
+    # logits of experts the router did not have to recompute exactly are its
+    # first-pass values: 2e-6, or two float steps of the value where that is more
+    np.testing.assert_allclose(R["score"][act], score[act], rtol=2.0 ** -22, atol=2e-6)
     np.testing.assert_allclose(R["topk_v"], tv, rtol=0, atol=1e-6)
     assert np.array_equal(R["offsets"], off), "offsets differ"
     assert np.array_equal(R["perm"][:off[-1]], perm), "per-expert permutation differs"
@@ -51,12 +53,12 @@ def check_routing(R, L, x, pos, E):
     return ti, off
 
 
-def stratified_rows(R, E, cap=640, seed=0):
+def stratified_rows(R, E, cap=640, seed=0, at_least=0):
     """Token rows that cover the GEMMs' tile plan: for every expert one row out
     of each of its row blocks of 32 (always from the first and the last block, so
     every row-block position of every tile height is hit, the ragged last block
     included), at varying places inside the block, thinned evenly down to about
-    `cap` tokens."""
+    `cap` tokens and topped up with random tokens to `at_least`."""
     off, perm = R["offsets"], R["perm"]
     must, rest = [], []
     for e in range(E):
@@ -73,7 +75,12 @@ def stratified_rows(R, E, cap=640, seed=0):
     room = max(cap - len(must), 0)
     if len(rest) > room:
         rest = list(np.random.default_rng(seed).choice(rest, room, replace=False))
-    return np.array(sorted(set(must) | set(int(t) for t in rest)), dtype=np.int64)
+    rows = set(must) | set(int(t) for t in rest)
+    if len(rows) < at_least:
+        T = len(perm) // 4
+        others = np.setdiff1d(np.arange(T), np.fromiter(rows, dtype=np.int64))
+        rows |= set(int(t) for t in np.random.default_rng(seed + 1).choice(others, at_least - len(rows), replace=False))
+    return np.array(sorted(rows), dtype=np.int64)
 
 
 def check_outputs(R, L, x, pos, rows, limit=7.0):
@@ -195,7 +202,7 @@ def test_c2_full_batch(c2):
     _, off = check_routing(R, L, L["x"], None, sh.experts)
     counts = np.diff(off)
     assert counts.sum() == 4 * T and counts.min() > 300  # roughly uniform load
-    rows = stratified_rows(R, sh.experts)
+    rows = stratified_rows(R, sh.experts, at_least=512)
     assert len(rows) >= 512
     err = check_outputs(R, L, L["x"], None, rows)
     print(f"c2 rel-L2 vs oracle on {len(rows)} rows: {err:.2e}; rows per expert {counts.min()}..{counts.max()}")
@@ -263,7 +270,8 @@ def test_c3_zipf_routing(name, c2):
         counts = np.diff(off)
         print(f"{name}: rows per expert max {counts.max()} min {counts.min()} (T={sh.tokens})")
         assert counts.max() > 6 * max(counts.min(), 1)  # the load really is skewed
-        rows = stratified_rows(R, sh.experts, cap=640 if name == "c3b" else 200)
+        rows = stratified_rows(R, sh.experts, cap=640 if name == "c3b" else 200,
+                               at_least=512 if name == "c3b" else 64)
         assert len(rows) >= (512 if name == "c3b" else 64)
         check_outputs(R, L, x, None, rows)
     finally:
@@ -326,7 +334,7 @@ def test_c4_120b_shape():
     m = make_moe(sh, L, sh.tokens)
     R = abi.run_layer(m, 0, L["x"], None)
     check_routing(R, L, L["x"], None, sh.experts)
-    rows = stratified_rows(R, sh.experts)
+    rows = stratified_rows(R, sh.experts, at_least=512)
     assert len(rows) >= 512
     check_outputs(R, L, L["x"], None, rows)
     # the large-batch GEMMs at 128 experts, twelve calls: same bits every time

@@ -122,7 +122,9 @@ def _check_ids(m, L, x, pos, E):
     assert np.array_equal(R["topk_i"], ti), "expert ids differ from the oracle"
     np.testing.assert_allclose(R["topk_v"], tv, rtol=0, atol=1e-6)
     act = np.ones(x.shape[0], bool) if pos is None else pos >= 0
-    np.testing.assert_allclose(R["score"][act], score[act], rtol=0, atol=2e-6)
+    # logits of experts the router did not have to recompute exactly are its
+    # first-pass values: 2e-6, or two float steps of the value where that is more
+    np.testing.assert_allclose(R["score"][act], score[act], rtol=2.0 ** -22, atol=2e-6)
     return R, score, ti
 
 
@@ -170,7 +172,7 @@ def test_router_first_pass_error_bound():
     x = synth.round_bf16(L["x"] * np.random.default_rng(1).uniform(0.1, 30.0, (T, 1)).astype(np.float32))
     m = make_moe(sh, L, T)
     R, score, _ = _check_ids_loose(m, L, x, E)
-    gamma = 2.0 * 33.0 * 4 * 2.0 ** -23
+    gamma = 2.0 * 33.0 * 2.0 ** -23  # router_gamma(1): a hand-over to fp64 after every MFMA
     bound = gamma * np.linalg.norm(x.astype(np.float64), axis=1) * np.linalg.norm(
         L["w_router"].astype(np.float64), axis=1).max()
     ratio = np.abs(R["score"].astype(np.float64) - score).max(axis=1) / bound
