@@ -23,7 +23,7 @@ SYMBOLS = [
     "moe_forward", "moe_block_forward",
     "moe_router",
     "moe_dispatch", "moe_get_dispatch", "moe_experts", "moe_expert_gemms", "moe_combine",
-    "moe_profile_enable",
+    "moe_dispatch_static", "moe_profile_enable",
     "moe_profile_read", "moe_weight_bytes", "moe_workspace_bytes", "moe_last_error",
     "moe_version", "moe_dev_alloc", "moe_dev_free", "moe_dev_upload", "moe_dev_download",
     "moe_dev_memset", "moe_dev_sync", "moe_dev_count", "moe_time_forward",
@@ -66,6 +66,7 @@ def lib() -> C.CDLL:
         L.moe_experts.argtypes = [vp, ci, vp, vp, vp, vp, ci, vp, ci, vp]
         L.moe_expert_gemms.argtypes = [vp, ci, vp, ci, vp]
         L.moe_combine.argtypes = [vp, vp, vp, ci, vp, ci, vp]
+        L.moe_dispatch_static.argtypes = [vp, vp, ci, ci, vp, vp, vp]
         L.moe_profile_enable.argtypes = [vp, ci]
         L.moe_profile_read.argtypes = [vp, C.POINTER(cf), C.POINTER(ci)]
         L.moe_weight_bytes.argtypes = [vp]
@@ -133,6 +134,12 @@ class DevBuf:
             self.close()
         except Exception:
             pass
+
+
+def dispatch_static(topk_i, pos, n_tokens, n_experts, offsets, perm, stream=None) -> None:
+    """moe_dispatch_static: no handle, no allocation; device buffers in and out."""
+    check(lib().moe_dispatch_static(_p(topk_i), _p(pos), n_tokens, n_experts, _p(offsets), _p(perm),
+                                    stream))
 
 
 def sync() -> None:

@@ -549,3 +549,89 @@ hipError_t launch_combine_residual(const float *y, const int *inv, const float *
 }
 
 }  // namespace moe
+
+// ---- dispatch for callers that cannot allocate ----
+//
+// moe_dispatch_static runs the same kernels as moe_dispatch, but needs no
+// handle and calls no allocating routine: the buffers the kernels use beyond
+// the caller's inputs and outputs (per-workgroup counts, the padded row map,
+// the inverse map, the per-expert records and the plan's totals) live in one
+// file-scope device array.  Every GPU the library runs on holds that array
+// until the process ends; every call on a GPU shares it, so calls that overlap
+// on one GPU (two streams, two threads) race.  The kernels rewrite everything
+// they later read, so nothing of an earlier call survives into the next.
+namespace moe {
+namespace {
+
+constexpr int kStaticMaxTokens = MOE_DISPATCH_STATIC_MAX_TOKENS;
+constexpr int kStaticMaxExperts = MOE_DISPATCH_STATIC_MAX_EXPERTS;
+constexpr size_t align256(size_t n) { return (n + 255) & ~(size_t)255; }
+constexpr size_t kStaticBlkCounts = 0;
+constexpr size_t kStaticRowmap =
+    kStaticBlkCounts + align256(sizeof(int) * ((kStaticMaxTokens + kDispThreads - 1) / kDispThreads) * kStaticMaxExperts);
+constexpr int kStaticPadRows = kStaticMaxTokens * kTopK + kTileGran * kStaticMaxExperts;
+constexpr size_t kStaticInv = kStaticRowmap + align256(sizeof(int) * kStaticPadRows);
+constexpr size_t kStaticInfo = kStaticInv + align256(sizeof(int) * kStaticMaxTokens * kTopK);
+constexpr size_t kStaticTotals = kStaticInfo + align256(sizeof(ExpertInfo) * kStaticMaxExperts);
+constexpr size_t kStaticBytes = kStaticTotals + align256(sizeof(int) * kTotInts);
+
+static __device__ __align__(256) unsigned char scratch[kStaticBytes];
+
+// Device address of this GPU's copy of `scratch`: looked up once per device
+// (each GPU holds its own copy at its own address), never taken from the
+// array's name, which on the host is only a stand-in for the symbol.
+constexpr int kMaxDevices = 64;
+unsigned char *g_scratch_ptr[kMaxDevices];  // written once per device, then only read
+
+hipError_t static_scratch(unsigned char **out) {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return e;
+  if (dev < 0 || dev >= kMaxDevices) return hipErrorInvalidDevice;
+  unsigned char *p = __atomic_load_n(&g_scratch_ptr[dev], __ATOMIC_ACQUIRE);
+  if (!p) {
+    e = hipGetSymbolAddress(reinterpret_cast<void **>(&p), HIP_SYMBOL(scratch));
+    if (e != hipSuccess) return e;
+    if (!p) return hipErrorInvalidSymbol;
+    __atomic_store_n(&g_scratch_ptr[dev], p, __ATOMIC_RELEASE);  // the same value from every thread
+  }
+  *out = p;
+  return hipSuccess;
+}
+
+}  // namespace
+}  // namespace moe
+
+extern "C" int moe_dispatch_static(const int *topk_i, const int *pos, int n_tokens, int n_experts,
+                                   int *offsets, int *perm, void *stream) {
+  using namespace moe;
+  if (n_tokens < 0) return set_error(MOE_ERR_BAD_ARG, "n_tokens %d is negative", n_tokens);
+  if (n_tokens > kStaticMaxTokens)
+    return set_error(MOE_ERR_CAPACITY, "moe_dispatch_static: n_tokens %d exceeds its fixed maximum of %d",
+                     n_tokens, kStaticMaxTokens);
+  if (n_experts < 1 || n_experts > kStaticMaxExperts)
+    return set_error(MOE_ERR_CAPACITY, "moe_dispatch_static: n_experts %d outside [1,%d]", n_experts,
+                     kStaticMaxExperts);
+  if (!offsets || (n_tokens > 0 && (!topk_i || !perm)))
+    return set_error(MOE_ERR_BAD_ARG, "null device pointer");
+  unsigned char *base = nullptr;
+  const hipError_t e = static_scratch(&base);
+  if (e != hipSuccess)
+    return set_error(MOE_ERR_HIP, "hipGetSymbolAddress(scratch) failed: %s", hipGetErrorString(e));
+  DispatchBuffers d{};
+  d.blk_counts = reinterpret_cast<int *>(base + kStaticBlkCounts);
+  d.rowmap = reinterpret_cast<int *>(base + kStaticRowmap);
+  d.inv = reinterpret_cast<int *>(base + kStaticInv);
+  d.info = reinterpret_cast<ExpertInfo *>(base + kStaticInfo);
+  d.totals = reinterpret_cast<int *>(base + kStaticTotals);
+  d.offsets = offsets;
+  d.perm = perm;
+  d.a_pad_cap = kStaticPadRows;
+  // no GEMM follows: with no column tiles the plan kernel writes no tile tables
+  d.tiles_gate_up = d.tiles_down = nullptr;
+  d.tile_cap_gate_up = d.tile_cap_down = 0;
+  const hipError_t el = launch_dispatch(topk_i, pos, n_tokens, n_experts, 0, 0, d, static_cast<hipStream_t>(stream));
+  if (el != hipSuccess)
+    return set_error(MOE_ERR_HIP, "dispatch launch failed: %s", hipGetErrorString(el));
+  return MOE_OK;
+}

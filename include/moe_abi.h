@@ -167,6 +167,25 @@ int moe_experts(moe_handle *h, int layer, const uint16_t *x, const int *pos,
                 const int *topk_i, const float *topk_v, int n_tokens,
                 float *out, int accumulate, void *stream);
 
+/* moe_dispatch for callers that cannot allocate device memory: code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc.  It has
+ * no counterpart in the reference.  No handle is needed and no allocating
+ * routine is called: the kernels' working buffers live in a device array that
+ * is part of the library image (about 330 KB per GPU, held until the process
+ * ends).  Inputs as moe_dispatch; the results go to the caller's device
+ * buffers offsets int [n_experts+1] and perm int [n_tokens*K] (entries past
+ * offsets[n_experts] are -1), bit-identical to moe_dispatch + moe_get_dispatch.
+ * Limits: n_tokens <= MOE_DISPATCH_STATIC_MAX_TOKENS, n_experts <=
+ * MOE_DISPATCH_STATIC_MAX_EXPERTS, otherwise MOE_ERR_CAPACITY.  All calls on
+ * one GPU share the array: calls that overlap on one GPU (two streams, two
+ * threads) race; calls on one stream are ordered.  The first call on a device
+ * looks up the array's address (hipGetSymbolAddress); make it outside a graph
+ * capture. */
+#define MOE_DISPATCH_STATIC_MAX_TOKENS 8192
+#define MOE_DISPATCH_STATIC_MAX_EXPERTS 256
+int moe_dispatch_static(const int *topk_i, const int *pos, int n_tokens,
+                        int n_experts, int *offsets, int *perm, void *stream);
+
 /* Stages 3-5 alone, on the plan of the last moe_dispatch of the same batch:
  * gathers the routed rows of x into per-expert segments, runs the gate_up
  * grouped GEMM with the clamped SwiGLU and the down grouped GEMM, and leaves one
