@@ -4,12 +4,12 @@
 
 A step is one moe_forward over one batch of synthetic input already resident in
 HBM.  Prints ONE JSON line: MoE-layer tokens/s, the roofline of the dominant
-kernel (gate_up grouped GEMM, priced against the dense bf16 MFMA peak) from HIP
-events recorded inside the timed steps, and the CPU baseline (the oracle's
-restatement of the reference's CPU/OpenMP path) timed on this host on a bounded
-prefix of the same batch.  At the default workload the line also carries
-"decode_mxfp4", a side figure for the decode-regime configuration (64 tokens,
-MXFP4 expert weights) priced against the HBM peak; `--workload c5` makes that
+kernel (the gate_up grouped GEMM) priced against whichever of the dense bf16
+MFMA peak and the HBM peak binds the workload, from HIP events recorded inside
+the timed steps, and the CPU baseline (the reference's CPU/OpenMP path) timed on
+this host on a bounded prefix of the same batch.  At the default workload the
+line also carries "decode_mxfp4", a side figure for the decode-regime
+configuration (64 tokens, MXFP4 expert weights); `--workload c5` makes that
 configuration the one measured.
 """
 from __future__ import annotations
@@ -17,6 +17,7 @@ from __future__ import annotations
 import argparse
 import json
 import os
+import re
 import sys
 import time
 
@@ -27,64 +28,100 @@ sys.path.insert(0, ROOT)
 
 PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0
-# What the box itself reaches with no algorithm in the way (second denominators,
-# reported next to the published peaks): v_mfma_f32_32x32x16_bf16 from registers
-# on all 256 CUs (profiles/mfma_register_rate.md) and a plain read stream over
-# 2 GB (profiles/l2_ingest_ceiling.md).
 SETTLE_STEPS = 200  # untimed calls in front of the warm-up steps, see run_leg
-MEASURED_MFMA_TFLOPS = 1880.0
-MEASURED_HBM_STREAM_GBS = 6150.0
-
-# HBM bytes per gate_up launch at the c2 workload from rocprofv3 --pmc
-# (FETCH_SIZE + WRITE_SIZE, scaled by the same counters on a copy kernel);
-# None until measured for the workload being run.
-MEASURED_TRAFFIC_BYTES = {"c2": 1.70e9, "c5": 0.290e9}  # profiles/bench_c2_counters.md, bench_c5_mxfp4_decode.md
+# which roofline binds the gate_up GEMM of a workload: rows per expert
+# (4 T / E) against the machine balance of 312 flop per byte
+BOUND = {"c2": "mfma", "c3a": "hbm", "c3b": "mfma", "c4": "hbm", "c5": "hbm"}
 
 
-def cpu_baseline(shape, L, budget_s=15.0):
+def cpu_model() -> str:
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("model name"):
+                return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
+def measured_traffic(workload: str):
+    """HBM bytes per gate_up launch from the rocprofv3 --pmc summary of this
+    workload under profiles/ (FETCH_SIZE + WRITE_SIZE, scaled by the same
+    counters on a copy of known size), or None where no such summary exists.
+    Read at run time so that the figure is the profile's, never a constant here."""
+    path = os.path.join(ROOT, "profiles", f"bench_{workload}_counters.md")
+    try:
+        m = re.search(r"gate_up traffic bytes per launch:\s*([0-9.eE+]+)", open(path).read())
+        return float(m.group(1)) if m else None
+    except OSError:
+        return None
+
+
+def cpu_baseline(shape, L, budget_s=12.0):
     """Times the reference's CPU path (per-token GEMV, OpenMP over output rows,
     float products accumulated in double; run.cpp:356-369, :662-745) on a prefix
-    of the batch sized for about budget_s seconds: the reference's own forward()
-    compiled from its sources (oracle/_ref, kind "reference") where that library
-    is there and loads, otherwise the oracle's restatement of it (kind "port")."""
+    of the batch sized for about budget_s seconds.  kind "reference": the
+    reference's own forward() compiled from its sources (oracle/_ref: -O3
+    -fopenmp, built where the sources are, hence without -march=native).  The
+    restatement of the same path, compiled on this host with the reference's
+    flags (-O3 -fopenmp -march=native), is timed next to it ("port_value").
+    Where oracle/_ref is missing the restatement is the baseline (kind "port")."""
     from oracle import binding as ob
     w = [L[k] for k in ("w_router", "b_router", "w_mlp1", "b_mlp1", "w_mlp2", "b_mlp2")]
     x = L["x"]
+    native = ob.lib_native()
 
     def port(rows):
-        ob.moe_layer(np.ascontiguousarray(x[:rows]), None, *w, shape.topk, shape.limit, mode=0)
+        ob.moe_layer(np.ascontiguousarray(x[:rows]), None, *w, shape.topk, shape.limit, mode=0, use_lib=native)
 
     def reference(rows):
         # forward() normalises its input row itself (unit norm weight): feed rows
         # of the same scale; the work does not depend on the values
         ob.ref_moe_forward(np.ascontiguousarray(x[:rows]), *w, shape.topk, shape.limit)
 
-    kind, run = "port", port
+    def timed(run, share):
+        n0 = min(8, x.shape[0])
+        t0 = time.perf_counter()
+        run(n0)
+        per_tok = (time.perf_counter() - t0) / n0
+        n = int(max(16, min(x.shape[0], 2048, share / max(per_tok, 1e-6))))
+        t0 = time.perf_counter()
+        run(n)
+        dt = time.perf_counter() - t0
+        return n / dt, n, dt
+
+    have_ref = False
     if ob.ref_available():
         try:
             reference(1)
-            kind, run = "reference", reference
-        except Exception:  # the library does not load on this host: time the restatement
-            pass
-    n0 = min(8, x.shape[0])
-    t0 = time.perf_counter()
-    run(n0)
-    per_tok = (time.perf_counter() - t0) / n0
-    n = int(max(16, min(x.shape[0], 2048, budget_s / max(per_tok, 1e-6))))
-    t0 = time.perf_counter()
-    run(n)
-    dt = time.perf_counter() - t0
-    return {"value": n / dt, "unit": "tokens/s", "cores": ob.num_threads(), "kind": kind,
-            "sample": f"first {n} of {x.shape[0]} tokens, fp32 host weights, {dt:.1f} s"}
+            have_ref = True
+        except Exception as e:  # the library does not load on this host
+            print(f"oracle/_ref does not load here ({e}); timing the restatement", file=sys.stderr)
+    pv, pn, pdt = timed(port, budget_s * (0.4 if have_ref else 1.0))
+    out = {"unit": "tokens/s", "cores": ob.num_threads(), "cpu": cpu_model()}
+    if have_ref:
+        rv, rn, rdt = timed(reference, budget_s * 0.6)
+        out.update({"value": rv, "kind": "reference",
+                    "sample": f"first {rn} of {x.shape[0]} tokens, fp32 host weights, {rdt:.1f} s",
+                    "flags": "-O3 -fopenmp (reference sources; built off this host, so without -march=native)",
+                    "port_value": pv,
+                    "port_sample": f"first {pn} tokens, {pdt:.1f} s; -O3 -fopenmp -march=native, built on this host"})
+    else:
+        out.update({"value": pv, "kind": "port",
+                    "sample": f"first {pn} of {x.shape[0]} tokens, fp32 host weights, {pdt:.1f} s",
+                    "flags": "-O3 -fopenmp -march=native, built on this host"})
+    return out
 
 
 def run_leg(shape, steps, warmup, device_timed=False):
     """Uploads the workload's layer, runs `warmup` + `steps` forwards and returns
     (seconds per step, stage times in ms from HIP events in the timed steps,
-    calls measured, host-side layer or None).  Seconds per step are wall-clock
-    time around the steps between two synchronisations; device_timed takes them
-    from two HIP events around the steps enqueued by one library call instead (a
-    step of 150 us is otherwise timed by the interpreter's call overhead)."""
+    calls measured, median seconds per step, host-side layer or None).  Seconds
+    per step are wall-clock time around the steps between two synchronisations;
+    device_timed takes them from two HIP events around the steps enqueued by one
+    library call instead (a step of 150 us is otherwise timed by the
+    interpreter's call overhead).  The median is over per-step HIP-event
+    intervals of a further run of max(steps, 50) steps."""
     from gpt_oss_amd import abi, synth
     T, H, IM, E = shape.tokens, shape.hidden, shape.inter, shape.experts
     moe = abi.Moe(H, IM, E, max_tokens=T, swiglu_limit=shape.limit)
@@ -121,8 +158,9 @@ def run_leg(shape, steps, warmup, device_timed=False):
     stages, n_meas = moe.profile_read()
     if device_timed:
         elapsed = moe.time_forward(0, dx, None, T, dout, warmup, steps) * 1e-3
+    each = moe.time_forward_each(0, dx, None, T, dout, max(steps, 50))
     moe.close()
-    return elapsed / steps, stages, n_meas, L
+    return elapsed / steps, stages, n_meas, float(np.median(each)) * 1e-3, L
 
 
 def mxfp4_weight_bytes(shape):
@@ -153,29 +191,34 @@ def main():
     shape = synth.CONFIGS[args.workload]
     T, H, IM, E, K = shape.tokens, shape.hidden, shape.inter, shape.experts, shape.topk
     mxfp4 = shape.name == "c5"
-    s_per_step, stages, n_meas, L = run_leg(shape, args.steps, args.warmup)
+    s_per_step, stages, n_meas, median_s, L = run_leg(shape, args.steps, args.warmup)
 
     A = T * K
     flops_gate_up = 2.0 * A * H * 2 * IM
     flops_down = 2.0 * A * IM * H
-    both = (flops_gate_up + flops_down) / ((stages["gate_up"] + stages["down"]) * 1e-3) / 1e12
+    t_gate_up = stages["gate_up"] * 1e-3
+    t_gemms = (stages["gate_up"] + stages["down"]) * 1e-3
+    both = (flops_gate_up + flops_down) / t_gemms / 1e12
+    w_elem = (0.5 + 1.0 / 32) if mxfp4 else 2.0  # bytes per expert weight in HBM
+    # algorithmic bytes: every expert matrix once, routed rows in, activations / fp32 rows out
+    bytes_gate_up = E * 2 * IM * H * w_elem + A * H * 2 + A * IM * 2
+    bytes_down = E * H * IM * w_elem + A * IM * 2 + A * H * 4
     router_bytes = T * H * 2 + E * H * 2 + E * 2 + T * K * 8
+    dispatch_bytes = T * K * 4 + A * 4 + (E + 1) * 4
     combine_bytes = A * H * 2 + T * H * 4
-    if mxfp4:
-        # a stream of weights: gate_up reads two thirds of them
-        achieved = mxfp4_weight_bytes(shape) * 2 / 3 / (stages["gate_up"] * 1e-3) / 1e9
-        roofline = {"bound": "hbm", "kernel": "grouped_gemm_kernel<gate_up, MXFP4>",
-                    "achieved": achieved, "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                    "frac": achieved / PEAK_HBM_GBS, "traffic": MEASURED_TRAFFIC_BYTES.get(shape.name),
-                    "measured_peak": MEASURED_HBM_STREAM_GBS,
-                    "frac_of_measured_peak": achieved / MEASURED_HBM_STREAM_GBS}
+    mfma_tflops = flops_gate_up / t_gate_up / 1e12
+    hbm_gbs = bytes_gate_up / t_gate_up / 1e9
+    kernel = "grouped_gemm_kernel<gate_up%s>" % (", MXFP4" if mxfp4 else "")
+    if BOUND[shape.name] == "mfma":
+        roofline = {"bound": "mfma", "kernel": kernel, "achieved": mfma_tflops, "peak": PEAK_BF16_TFLOPS,
+                    "unit": "TFLOP/s", "frac": mfma_tflops / PEAK_BF16_TFLOPS}
     else:
-        achieved = flops_gate_up / (stages["gate_up"] * 1e-3) / 1e12
-        roofline = {"bound": "mfma", "kernel": "grouped_gemm_kernel<gate_up>",
-                    "achieved": achieved, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                    "frac": achieved / PEAK_BF16_TFLOPS, "traffic": MEASURED_TRAFFIC_BYTES.get(shape.name),
-                    "measured_peak": MEASURED_MFMA_TFLOPS,
-                    "frac_of_measured_peak": achieved / MEASURED_MFMA_TFLOPS}
+        roofline = {"bound": "hbm", "kernel": kernel, "achieved": hbm_gbs, "peak": PEAK_HBM_GBS,
+                    "unit": "GB/s", "frac": hbm_gbs / PEAK_HBM_GBS}
+    roofline["traffic"] = measured_traffic(shape.name)
+    # the other roofline of the same kernel, for the workloads near the machine balance
+    roofline["frac_mfma_peak"] = mfma_tflops / PEAK_BF16_TFLOPS
+    roofline["frac_hbm_peak"] = hbm_gbs / PEAK_HBM_GBS
     weights = "MXFP4 expert weights" if mxfp4 else "bf16 weights"
     result = {
         "metric": "MoE-layer tokens/sec",
@@ -186,6 +229,7 @@ def main():
         "warmup": args.warmup,
         "settle_steps": SETTLE_STEPS,
         "ms_per_step": s_per_step * 1e3,
+        "median_ms_per_step": median_s * 1e3,
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
@@ -194,9 +238,12 @@ def main():
         "config": {"workload": f"{shape.name}: {T} tokens, hidden {H}, intermediate {IM}, "
                                f"{E} experts, top-{K}, {weights}, fp32 accumulate, seed 0"},
         "roofline": roofline,
-        "expert_gemms": {"tflops": both, "frac_bf16_peak": both / PEAK_BF16_TFLOPS},
+        "expert_gemms": {"tflops": both, "frac_bf16_peak": both / PEAK_BF16_TFLOPS,
+                         "gbs": (bytes_gate_up + bytes_down) / t_gemms / 1e9,
+                         "frac_hbm_peak": (bytes_gate_up + bytes_down) / t_gemms / 1e9 / PEAK_HBM_GBS},
         "stage_us": {k: v * 1e3 for k, v in stages.items()},
         "router_gbs": router_bytes / (stages["router"] * 1e-3) / 1e9,
+        "dispatch_gbs": dispatch_bytes / (stages["dispatch"] * 1e-3) / 1e9,
         "combine_gbs": combine_bytes / (stages["combine"] * 1e-3) / 1e9,
         "events_calls": n_meas,
     }
@@ -204,12 +251,12 @@ def main():
         # Side figure, not the headline value: the decode-regime configuration,
         # priced against the HBM peak on the weight bytes its GEMMs stream.
         c5 = synth.CONFIGS["c5"]
-        s5, st5, _, _ = run_leg(c5, 200, 20, device_timed=True)
+        s5, st5, _, med5, _ = run_leg(c5, 200, 20, device_timed=True)
         wb = mxfp4_weight_bytes(c5)
         gemm_s = (st5["gate_up"] + st5["down"]) * 1e-3
         result["decode_mxfp4"] = {
             "workload": f"c5: {c5.tokens} tokens, {c5.experts} experts, MXFP4 expert weights",
-            "tokens_per_s": c5.tokens / s5, "us_per_step": s5 * 1e6,
+            "tokens_per_s": c5.tokens / s5, "us_per_step": s5 * 1e6, "median_us_per_step": med5 * 1e6,
             "stage_us": {k: v * 1e3 for k, v in st5.items()},
             "weight_bytes": wb, "gemm_gbs": wb / gemm_s / 1e9,
             "gemm_frac_hbm_peak": wb / gemm_s / 1e9 / PEAK_HBM_GBS,

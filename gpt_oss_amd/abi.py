@@ -26,7 +26,7 @@ SYMBOLS = [
     "moe_dispatch_static", "moe_profile_enable",
     "moe_profile_read", "moe_weight_bytes", "moe_workspace_bytes", "moe_last_error",
     "moe_version", "moe_dev_alloc", "moe_dev_free", "moe_dev_upload", "moe_dev_download",
-    "moe_dev_memset", "moe_dev_sync", "moe_dev_count", "moe_time_forward",
+    "moe_dev_memset", "moe_dev_sync", "moe_dev_count", "moe_time_forward", "moe_time_forward_each",
 ]
 
 
@@ -81,6 +81,7 @@ def lib() -> C.CDLL:
         L.moe_dev_download.argtypes = [vp, vp, C.c_size_t]
         L.moe_dev_memset.argtypes = [vp, ci, C.c_size_t]
         L.moe_time_forward.argtypes = [vp, ci, vp, vp, ci, vp, ci, ci, C.POINTER(cf)]
+        L.moe_time_forward_each.argtypes = [vp, ci, vp, vp, ci, vp, ci, C.POINTER(cf)]
         _lib = L
     return _lib
 
@@ -233,6 +234,12 @@ class Moe:
         check(lib().moe_time_forward(self.h, layer, _p(x), _p(pos), n_tokens, _p(out), warmup,
                                      iters, C.byref(ms)))
         return float(ms.value)
+
+    def time_forward_each(self, layer, x, pos, n_tokens, out, iters) -> np.ndarray:
+        """Durations in ms of `iters` consecutive forward calls (HIP events on one stream)."""
+        ms = (C.c_float * iters)()
+        check(lib().moe_time_forward_each(self.h, layer, _p(x), _p(pos), n_tokens, _p(out), iters, ms))
+        return np.array(ms[:], dtype=np.float64)
 
     @property
     def weight_bytes(self):

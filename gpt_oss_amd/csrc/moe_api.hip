@@ -664,4 +664,29 @@ int moe_time_forward(moe_handle *h, int layer, const uint16_t *x, const int *pos
   return rc;
 }
 
+int moe_time_forward_each(moe_handle *h, int layer, const uint16_t *x, const int *pos, int n_tokens,
+                          float *out, int iters, float *ms_each) {
+  if (!ms_each || iters <= 0 || iters > 4096) return fail(MOE_ERR_BAD_ARG, "bad timing arguments");
+  hipStream_t s = nullptr;
+  HIP_TRY(hipStreamCreate(&s));
+  std::vector<hipEvent_t> ev((size_t)iters + 1, nullptr);
+  auto body = [&]() -> int {
+    for (auto &e : ev) HIP_TRY(hipEventCreate(&e));
+    HIP_TRY(hipEventRecord(ev[0], s));
+    for (int i = 0; i < iters; i++) {
+      int r = moe_forward(h, layer, x, pos, n_tokens, out, 0, s);
+      if (r != MOE_OK) return r;
+      HIP_TRY(hipEventRecord(ev[i + 1], s));
+    }
+    HIP_TRY(hipEventSynchronize(ev[iters]));
+    for (int i = 0; i < iters; i++) HIP_TRY(hipEventElapsedTime(&ms_each[i], ev[i], ev[i + 1]));
+    return MOE_OK;
+  };
+  const int rc = body();
+  for (hipEvent_t e : ev)
+    if (e) (void)hipEventDestroy(e);
+  (void)hipStreamDestroy(s);
+  return rc;
+}
+
 }  // extern "C"

@@ -122,12 +122,38 @@ static void mi355_moe_cleanup(DeviceContext &ctx) {
 }
 
 #ifdef MI355_MOE_REPLACE_EP
-// Keeps the reference's own names for a runner that calls the EP entry points
-// (getp_run.cpp:409, :435, :724) and no longer includes its own expert.cpp MoE.
+// The reference's own entry points (getp-csrc/expert.cpp) under their own names,
+// for a runner that takes its `use_expert_parallelism` branch (getp_run.cpp:408,
+// :434, :723) and whose expert.cpp no longer carries the MoE code -- see
+// shim/expert.cpp, which takes the place of that file.  One GPU: every expert is
+// local, so there is no exchange between devices.
+
+// init_device_context_ep (expert.cpp:709): everything that is not the MoE layer
+// (activations, attention and embedding weights, KV cache, streams) is set up by
+// the reference's own init_device_context (getp_run.cpp:19), defined further
+// down in the same translation unit; the expert weights go to libmi355_moe.
+static void init_device_context(DeviceContext &ctx, int device_id, Transformer *transformer);
+static void init_device_context_ep(DeviceContext &ctx, int device_id, Transformer *transformer) {
+  init_device_context(ctx, device_id, transformer);
+  mi355_moe_init(ctx, device_id, transformer, MAX_BATCH_SIZE);
+}
+
+// warm_up_ep (expert.cpp:1176): the reference builds its owner maps and enables
+// peer access here; with all experts on the one device only the per-device
+// initialisation is left (the same loop as expert.cpp:1216-1218).
+static void warm_up_ep(Transformer *transformer) {
+  for (int i = 0; i < g_num_devices; ++i) init_device_context_ep(g_devices[i], i, transformer);
+}
+
+// gpu_forward_device_batch_ep (expert.cpp:1366): same parameter list; the caller
+// has run the router and the top-k and zeroed d_e_agg (getp_run.cpp:697-720).
 static void gpu_forward_device_batch_ep(DeviceContext &ctx, const float swiglu_limit, const int H,
                                         const int IM, const int E, const int L, const int K,
                                         int batch_size, int layer) {
   mi355_moe_forward(ctx, swiglu_limit, H, IM, E, L, K, batch_size, layer);
 }
+
+// cleanup_device_context_ep (expert.cpp:1234): called by the reference's
+// cleanup_device_context after it has freed its own buffers (getp_run.cpp:408-410).
 static void cleanup_device_context_ep(DeviceContext &ctx) { mi355_moe_cleanup(ctx); }
 #endif

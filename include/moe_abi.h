@@ -238,6 +238,12 @@ int moe_time_forward(moe_handle *h, int layer, const uint16_t *x, const int *pos
                      int n_tokens, float *out, int warmup, int iters,
                      float *total_ms);
 
+/* The same with one HIP event after every call: ms_each[i] is the duration of
+ * call i (iters <= 4096), for the median the benchmark reports. */
+int moe_time_forward_each(moe_handle *h, int layer, const uint16_t *x,
+                          const int *pos, int n_tokens, float *out, int iters,
+                          float *ms_each);
+
 #ifdef __cplusplus
 }
 #endif

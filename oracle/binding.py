@@ -34,29 +34,43 @@ def _opt(a, dtype):
 _lib = None
 
 
+def _load(path):
+    L = C.CDLL(path)
+    L.oracle_f32_to_bf16.restype = C.c_uint16
+    L.oracle_f32_to_bf16.argtypes = [C.c_float]
+    L.oracle_bf16_to_f32.restype = C.c_float
+    L.oracle_bf16_to_f32.argtypes = [C.c_uint16]
+    L.oracle_round_to_bf16.argtypes = [_f, C.c_size_t]
+    L.oracle_matmul.argtypes = [_f, _f, _f, C.c_int, C.c_int]
+    L.oracle_topk.argtypes = [_f, _i, _f, C.c_int, C.c_int]
+    L.oracle_softmax.argtypes = [_f, C.c_int]
+    L.oracle_router.argtypes = [_f, C.c_void_p, _f, _f] + [C.c_int] * 4 + [_f, _i, _f]
+    L.oracle_dispatch.argtypes = [_i, C.c_void_p] + [C.c_int] * 3 + [_i, _i, C.c_void_p]
+    L.oracle_expert_token.argtypes = [_f] * 5 + [C.c_int, C.c_int, C.c_float, C.c_int, _f, _f]
+    L.oracle_moe_layer.argtypes = ([_f, C.c_void_p] + [_f] * 6 + [C.c_int] * 5 +
+                                       [C.c_float, C.c_int, _f, C.c_void_p, C.c_void_p, C.c_void_p])
+    L.oracle_mxfp4_dequant.argtypes = [_u8, _u8, C.c_size_t, _f]
+    L.oracle_rmsnorm.argtypes = [_f, _f, _f, C.c_int]
+    L.oracle_num_threads.restype = C.c_int
+    return L
+
+
 def lib():
     global _lib
     if _lib is None:
         build()
-        L = C.CDLL(os.path.join(_HERE, "liboracle.so"))
-        L.oracle_f32_to_bf16.restype = C.c_uint16
-        L.oracle_f32_to_bf16.argtypes = [C.c_float]
-        L.oracle_bf16_to_f32.restype = C.c_float
-        L.oracle_bf16_to_f32.argtypes = [C.c_uint16]
-        L.oracle_round_to_bf16.argtypes = [_f, C.c_size_t]
-        L.oracle_matmul.argtypes = [_f, _f, _f, C.c_int, C.c_int]
-        L.oracle_topk.argtypes = [_f, _i, _f, C.c_int, C.c_int]
-        L.oracle_softmax.argtypes = [_f, C.c_int]
-        L.oracle_router.argtypes = [_f, C.c_void_p, _f, _f] + [C.c_int] * 4 + [_f, _i, _f]
-        L.oracle_dispatch.argtypes = [_i, C.c_void_p] + [C.c_int] * 3 + [_i, _i, C.c_void_p]
-        L.oracle_expert_token.argtypes = [_f] * 5 + [C.c_int, C.c_int, C.c_float, C.c_int, _f, _f]
-        L.oracle_moe_layer.argtypes = ([_f, C.c_void_p] + [_f] * 6 + [C.c_int] * 5 +
-                                       [C.c_float, C.c_int, _f, C.c_void_p, C.c_void_p, C.c_void_p])
-        L.oracle_mxfp4_dequant.argtypes = [_u8, _u8, C.c_size_t, _f]
-        L.oracle_rmsnorm.argtypes = [_f, _f, _f, C.c_int]
-        L.oracle_num_threads.restype = C.c_int
-        _lib = L
+        _lib = _load(os.path.join(_HERE, "liboracle.so"))
     return _lib
+
+
+def lib_native():
+    """The restatement compiled on this host with -O3 -march=native -fopenmp (the
+    flags of the reference's OpenMP build); built on first use.  Used by the
+    benchmark's CPU-baseline leg only: the checker of the tests stays the
+    portable build."""
+    so = os.path.join(_HERE, "_native", "liboracle_native.so")
+    subprocess.check_call(["make", "-s", "-B", "-C", _HERE, "native"])
+    return _load(so)
 
 
 def f32_to_bf16(x: float) -> int:
@@ -119,7 +133,7 @@ def expert_token(t, w1, b1, w2, b2, limit, mode=0):
     return y
 
 
-def moe_layer(x, pos, wr, br, w1, b1, w2, b2, K, limit, mode=0, want_routing=False):
+def moe_layer(x, pos, wr, br, w1, b1, w2, b2, K, limit, mode=0, want_routing=False, use_lib=None):
     T, H = x.shape
     E = wr.shape[0]
     IM = w2.shape[2]
@@ -127,7 +141,7 @@ def moe_layer(x, pos, wr, br, w1, b1, w2, b2, K, limit, mode=0, want_routing=Fal
     score = np.zeros((T, E), np.float32) if want_routing else None
     ti = np.zeros((T, K), np.int32) if want_routing else None
     tv = np.zeros((T, K), np.float32) if want_routing else None
-    lib().oracle_moe_layer(x, _opt(pos, np.int32), wr, br, w1, b1, w2, b2, T, H, IM, E, K,
+    (use_lib or lib()).oracle_moe_layer(x, _opt(pos, np.int32), wr, br, w1, b1, w2, b2, T, H, IM, E, K,
                            limit, mode, out, _opt(score, np.float32), _opt(ti, np.int32),
                            _opt(tv, np.float32))
     return (out, score, ti, tv) if want_routing else out

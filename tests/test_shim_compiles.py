@@ -1,7 +1,12 @@
 """The C++17 host shim compiles against the reference's own types (Transformer,
-DeviceContext, Config) and links against the C-ABI library.  Needs the reference
-checkout, so it runs in the build container only.  No GPU."""
+DeviceContext, Config), and the reference's whole getp translation unit (run.cpp
+with getp-csrc/getp_run.cpp, no -DTESTING) compiles unmodified with
+shim/expert.cpp in the place of its getp-csrc/expert.cpp.  Needs the reference
+checkout, so these run in the build container only; the reference's files are
+copied into a temporary directory for the duration of the test and nothing of
+them is kept.  No GPU."""
 import os
+import shutil
 import subprocess
 import tempfile
 
@@ -9,6 +14,9 @@ import pytest
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 REF = "/root/reference"
+HIPCC = "/opt/rocm/bin/hipcc"
+needs_ref = pytest.mark.skipif(not os.path.exists(os.path.join(REF, "run.cpp")),
+                               reason="reference checkout not present")
 
 TU = r'''
 #define TESTING
@@ -22,18 +30,50 @@ void shim_smoke(Transformer *t) {
   mi355_moe_forward(ctx, p->swiglu_limit, p->hidden_dim, p->intermediate_dim, p->n_experts,
                     p->n_layers, p->experts_per_token, 1, 0);
   mi355_moe_forward_fused(ctx, 1, 0);
+  mi355_moe_block(ctx, 1, 0);
   mi355_moe_cleanup(ctx);
 }
 '''
 
 
-@pytest.mark.skipif(not os.path.exists(os.path.join(REF, "run.cpp")), reason="reference checkout not present")
+def _hipcc(args, cwd=None):
+    cmd = [HIPCC, "--std=c++17", "--offload-arch=gfx950", "-fopenmp", "-include", "thread", "-w",
+           "-I", os.path.join(ROOT, "include"), "-I", os.path.join(ROOT, "gpt_oss_amd", "shim")] + args
+    r = subprocess.run(cmd, capture_output=True, text=True, cwd=cwd)
+    assert r.returncode == 0, r.stderr[-3000:]
+
+
+@needs_ref
 def test_shim_compiles_against_reference_types():
     with tempfile.TemporaryDirectory() as d:
         src = os.path.join(d, "tu.cpp")
         open(src, "w").write(TU % {"ref": REF})
-        cmd = ["/opt/rocm/bin/hipcc", "--std=c++17", "--offload-arch=gfx950", "-fopenmp", "-include",
-               "thread", "-w", "-I", REF, "-I", os.path.join(ROOT, "include"), "-I",
-               os.path.join(ROOT, "gpt_oss_amd", "shim"), "-c", src, "-o", os.path.join(d, "tu.o")]
-        r = subprocess.run(cmd, capture_output=True, text=True)
-        assert r.returncode == 0, r.stderr[-3000:]
+        _hipcc(["-I", REF, "-c", src, "-o", os.path.join(d, "tu.o")])
+
+
+@needs_ref
+def test_reference_getp_unit_builds_with_replacement_expert_cpp():
+    """run.cpp -> getp-csrc/getp_run.cpp -> "expert.cpp" (getp_run.cpp:4), all
+    unmodified, with shim/expert.cpp as that file and the reference's own as
+    expert_ref.cpp: warm_up_ep, init_device_context_ep, gpu_forward_device_batch_ep
+    and cleanup_device_context_ep (getp_run.cpp:409, :435, :724) resolve to the
+    shim, and the object links against libmi355_moe with no MoE symbol missing."""
+    with tempfile.TemporaryDirectory() as d:
+        tree = os.path.join(d, "ref")
+        shutil.copytree(REF, tree, ignore=shutil.ignore_patterns(".git", "*.bin", "*.so", "*.o", "tests", "data",
+                                                                 "export_model_bin", "*.txt", "*.md"))
+        getp = os.path.join(tree, "getp-csrc")
+        os.rename(os.path.join(getp, "expert.cpp"), os.path.join(getp, "expert_ref.cpp"))
+        shutil.copy(os.path.join(ROOT, "gpt_oss_amd", "shim", "expert.cpp"), os.path.join(getp, "expert.cpp"))
+        obj = os.path.join(d, "run.o")
+        _hipcc(["-c", os.path.join(tree, "run.cpp"), "-o", obj], cwd=tree)
+        # the four entry points come from the shim: the renamed originals are still
+        # there (static, unused), the calls bind to moe_* of the C-ABI
+        nm = subprocess.run(["nm", "-C", "--undefined-only", obj], capture_output=True, text=True).stdout
+        for sym in ("moe_create", "moe_upload_layer", "moe_experts", "moe_destroy"):
+            assert sym in nm, f"{sym} is not referenced by the runner's object"
+        lib = os.path.join(ROOT, "gpt_oss_amd", "libmi355_moe.so")
+        if os.path.exists(lib):
+            tok = os.path.join(d, "tok.o")
+            _hipcc(["-c", os.path.join(tree, "tokenizer.cpp"), "-o", tok], cwd=tree)
+            _hipcc([obj, tok, "-L", os.path.dirname(lib), "-lmi355_moe", "-o", os.path.join(d, "run")])
