@@ -427,14 +427,17 @@ __global__ __launch_bounds__(kDispThreads) void dispatch_small_kernel(
 // (row block rb, k block kb) is 64 lanes x 16 bytes, lane l = row rb*32 + l%32,
 // k = 16*kb + 8*(l/32) .. +7.  Padding rows are zero.  One wave writes four
 // consecutive k blocks (4 KB) of one row block.
+constexpr int kGatherGridY = 32768;
 __global__ __launch_bounds__(256) void gather_rows_kernel(const uint16_t *__restrict__ x,
                                                          const int *__restrict__ rowmap,
                                                          const int *__restrict__ totals,
                                                          uint4 *__restrict__ xg, int H) {
-  const int rb = blockIdx.x;  // the x dimension of a grid has room for any batch the handle accepts
+  // row blocks run over the y and z dimensions of the grid (32768 each): room for
+  // any batch the handle accepts, with the k groups of a row block next to each other
+  const int rb = blockIdx.y + blockIdx.z * kGatherGridY;
   if (rb * kRowBlock >= totals[1]) return;
   const int lane = threadIdx.x & 63;
-  const int grp = blockIdx.y * 4 + (threadIdx.x >> 6);
+  const int grp = blockIdx.x * 4 + (threadIdx.x >> 6);
   const int kb_total = H / kFragK;
   if (grp * 4 >= kb_total) return;
   const int a = rowmap[rb * kRowBlock + (lane & 31)];
@@ -531,7 +534,7 @@ hipError_t launch_gather(const uint16_t *x, const DispatchBuffers &d, uint16_t *
                          int rb_cap, hipStream_t s) {
   (void)T;
   const int groups = H / 64;
-  dim3 grid(rb_cap, (groups + 3) / 4);
+  dim3 grid((groups + 3) / 4, rb_cap < kGatherGridY ? rb_cap : kGatherGridY, (rb_cap + kGatherGridY - 1) / kGatherGridY);
   gather_rows_kernel<<<grid, 256, 0, s>>>(x, d.rowmap, d.totals, reinterpret_cast<uint4 *>(xg), H);
   return hipGetLastError();
 }

@@ -22,7 +22,11 @@
 //     ring by DMA (global_load_lds_dwordx4), R-1 steps ahead of the MFMAs;
 //   * the column operand is private to a wave in this layout, so it never
 //     touches LDS: it is loaded into an R-slot ring of VGPRs, R-1 steps ahead.
-// With R = 7 that is 6 steps x 32 KB = 192 KB in flight per CU.  These loads
+// The full-height configuration runs R = 5 (4 steps x 32 KB = 128 KB in flight
+// per CU: measured against 6 and 7, a deeper ring gains nothing in the main loop
+// and costs the time its longer fill takes at the start of every tile, 0.8 % of
+// the layer at 4096 tokens); the small-batch configuration, a stream of weights
+// through two or three workgroups per CU, runs R = 7.  These loads
 // complete in the order they were issued, so waiting for "all but the newest n"
 // (s_waitcnt vmcnt(n)) picks out exactly the step that is needed next and
 // leaves the later ones in flight (the scattered DMA of the GATHER variant is
@@ -37,6 +41,7 @@
 // runs at one time share the expert's rows and a few column slabs of its
 // weights, so each weight byte leaves HBM once.
 #include <type_traits>
+#include <utility>
 
 #include "moe_internal.h"
 
@@ -44,6 +49,16 @@ namespace moe {
 
 template <int V>
 using IC = std::integral_constant<int, V>;
+
+// f(IC<0>{}), f(IC<1>{}), ..., f(IC<N-1>{})
+template <typename F, int... I>
+__device__ __forceinline__ void static_for_impl(F &&f, std::integer_sequence<int, I...>) {
+  (f(IC<I>{}), ...);
+}
+template <int N, typename F>
+__device__ __forceinline__ void static_for(F &&f) {
+  static_for_impl(f, std::make_integer_sequence<int, N>{});
+}
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
@@ -184,8 +199,11 @@ __device__ __forceinline__ void gemm_tile(const uint4 *__restrict__ a_frag,  // 
                                           // the epilogue's own stores included.
                                           uint4 *__restrict__ epi) {
   StageRing<C::R> ring;
-  ring.p[0] = s0; ring.p[1] = s1; ring.p[2] = s2; ring.p[3] = s3;
-  ring.p[4] = s4; ring.p[5] = s5; ring.p[6] = s6;
+  {
+    uint4 *const all[7] = {s0, s1, s2, s3, s4, s5, s6};
+#pragma unroll
+    for (int i = 0; i < C::R; i++) ring.p[i] = all[i];
+  }
   constexpr int NBW = C::NBW, KPS = C::KPS, R = C::R, NW = C::NW;
   static_assert(KPS == 2, "the step is software-pipelined as two k blocks");
   constexpr int A_CH = RBT * RS * KPS;       // 1 KB chunks of the row operand per step
@@ -323,7 +341,7 @@ __device__ __forceinline__ void gemm_tile(const uint4 *__restrict__ a_frag,  // 
       return __builtin_bit_cast(bf16x8, bq[slot][j * KPS + kk]);
     }
   };
-  static_assert(R == 7, "the step sequence below is written out for 7 slots");
+  static_assert(R >= 3 && R <= 7, "up to seven stage arrays are passed in");
   // "Step s of the row operand has landed" as a bound on the vector-memory
   // counter.  The loads are issued in the order A(0) B(0) A(1) B(1) ... and
   // complete in that order, so all but the newest n outstanding means step s has
@@ -432,21 +450,11 @@ __device__ __forceinline__ void gemm_tile(const uint4 *__restrict__ a_frag,  // 
     }
   };
   int ks0 = 0;
-  for (; ks0 + R <= n_steps; ks0 += R) {
-    step(IC<0>{}, ks0 + 0);
-    step(IC<1>{}, ks0 + 1);
-    step(IC<2>{}, ks0 + 2);
-    step(IC<3>{}, ks0 + 3);
-    step(IC<4>{}, ks0 + 4);
-    step(IC<5>{}, ks0 + 5);
-    step(IC<6>{}, ks0 + 6);
-  }
-  if (ks0 + 0 < n_steps) step(IC<0>{}, ks0 + 0);
-  if (ks0 + 1 < n_steps) step(IC<1>{}, ks0 + 1);
-  if (ks0 + 2 < n_steps) step(IC<2>{}, ks0 + 2);
-  if (ks0 + 3 < n_steps) step(IC<3>{}, ks0 + 3);
-  if (ks0 + 4 < n_steps) step(IC<4>{}, ks0 + 4);
-  if (ks0 + 5 < n_steps) step(IC<5>{}, ks0 + 5);
+  for (; ks0 + R <= n_steps; ks0 += R)
+    static_for<R>([&](auto u_c) { step(u_c, ks0 + decltype(u_c)::value); });
+  static_for<R - 1>([&](auto u_c) {
+    if (ks0 + decltype(u_c)::value < n_steps) step(u_c, ks0 + decltype(u_c)::value);
+  });
 
   // Epilogue.
   if (cw * NBW >= nb_valid) return;  // a wave without columns (last column tile only)
@@ -530,7 +538,7 @@ __global__ __launch_bounds__(C::THREADS, C::WAVES) void grouped_gemm_kernel(
     const int *__restrict__ rowmap, void *__restrict__ outp, int K, int N, float limit) {
   static_assert(!GATHER || GATE_UP, "only the first GEMM reads token rows");
   constexpr int R = C::R;
-  static_assert(R == 7, "seven stage arrays are declared below");
+  static_assert(R <= 7, "seven stage arrays are declared below");
   __shared__ uint4 st0[C::STAGE], st1[C::STAGE], st2[C::STAGE], st3[C::STAGE], st4[C::STAGE],
       st5[C::STAGE], st6[C::STAGE];
   __shared__ uint4 epi[C::NW * C::EPI_WAVE];
@@ -584,8 +592,8 @@ __global__ __launch_bounds__(C::THREADS, C::WAVES) void grouped_gemm_kernel(
 }
 
 // 4 waves, one per SIMD, each 256 rows x 64 columns (8 x 2 accumulators = all
-// 256 accumulation registers); 256 x 256 tiles; 7 ring slots.
-using CfgGemm = GemmCfg<4, 2, 7>;
+// 256 accumulation registers); 256 x 256 tiles; 5 ring slots.
+using CfgGemm = GemmCfg<4, 2, 5>;
 static_assert(CfgGemm::RBT_MAX * kRowBlock == kTileRows && CfgGemm::TILE_NB == kGemmTileNb,
               "tile plan of dispatch_scan_kernel");
 // Batches of at most 64 tokens: no expert has more than 64 rows, every tile is
