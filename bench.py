@@ -216,6 +216,8 @@ def main():
         roofline = {"bound": "hbm", "kernel": kernel, "achieved": hbm_gbs, "peak": PEAK_HBM_GBS,
                     "unit": "GB/s", "frac": hbm_gbs / PEAK_HBM_GBS}
     roofline["traffic"] = measured_traffic(shape.name)
+    roofline["traffic_source"] = (f"profiles/bench_{shape.name}_counters.md (rocprofv3 --pmc run of this workload, "
+                                  "not this run)" if roofline["traffic"] is not None else None)
     # the other roofline of the same kernel, for the workloads near the machine balance
     roofline["frac_mfma_peak"] = mfma_tflops / PEAK_BF16_TFLOPS
     roofline["frac_hbm_peak"] = hbm_gbs / PEAK_HBM_GBS
