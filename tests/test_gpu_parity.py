@@ -466,8 +466,7 @@ def test_forward_replays_from_a_hip_graph(c2, T):
     """moe_forward allocates nothing, never synchronises and clears its buffers
     with kernels, so a caller may capture it.  Three replays, with eager calls
     and synchronisations of the program's own in between, must each reproduce the
-    eager result bit for bit.  48 tokens take the small-batch kernels (the
-    arrival counters of the shared router tiles are reset by the kernel itself)."""
+    eager result bit for bit.  48 tokens take the small-batch kernels."""
     import ctypes as C
     hip = C.CDLL("libamdhip64.so")
 
