@@ -9,8 +9,9 @@ MFMA peak and the HBM peak binds the workload, from HIP events recorded inside
 the timed steps, and the CPU baseline (the reference's CPU/OpenMP path) timed on
 this host on a bounded prefix of the same batch.  At the default workload the
 line also carries "decode_mxfp4", a side figure for the decode-regime
-configuration (64 tokens, MXFP4 expert weights); `--workload c5` makes that
-configuration the one measured.
+configuration (64 tokens, MXFP4 expert weights; `--workload c5` makes that
+configuration the one measured), and "prefill_mxfp4", the headline batch with
+MXFP4 expert weights.  Neither is part of `value`.
 """
 from __future__ import annotations
 
@@ -113,7 +114,7 @@ def cpu_baseline(shape, L, budget_s=12.0):
     return out
 
 
-def run_leg(shape, steps, warmup, device_timed=False):
+def run_leg(shape, steps, warmup, device_timed=False, mxfp4=None):
     """Uploads the workload's layer, runs `warmup` + `steps` forwards and returns
     (seconds per step, stage times in ms from HIP events in the timed steps,
     calls measured, median seconds per step, host-side layer or None).  Seconds
@@ -125,7 +126,9 @@ def run_leg(shape, steps, warmup, device_timed=False):
     from gpt_oss_amd import abi, synth
     T, H, IM, E = shape.tokens, shape.hidden, shape.inter, shape.experts
     moe = abi.Moe(H, IM, E, max_tokens=T, swiglu_limit=shape.limit)
-    if shape.name == "c5":  # MXFP4 expert weights, read as MXFP4 by the GEMMs
+    if mxfp4 is None:
+        mxfp4 = shape.name == "c5"
+    if mxfp4:  # MXFP4 expert weights, read as MXFP4 by the GEMMs
         L = None
         wr, br = synth.make_router(shape)
         b1k, s1, b1, b2k, s2, b2 = synth.make_experts_mxfp4(shape)
@@ -176,7 +179,7 @@ def main():
     ap.add_argument("--workload", default="c2", help="c2 (headline), c3a, c3b, c4, c5 (MXFP4 decode)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-decode", action="store_true",
-                    help="c2 only: skip the decode-regime side figure (workload c5)")
+                    help="c2 only: skip the two side figures with MXFP4 weights (workload c5, and c2's batch)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)",
@@ -263,6 +266,20 @@ def main():
             "weight_bytes": wb, "gemm_gbs": wb / gemm_s / 1e9,
             "gemm_frac_hbm_peak": wb / gemm_s / 1e9 / PEAK_HBM_GBS,
             "layer_gbs": wb / s5 / 1e9}
+        # Second side figure: the headline batch with the expert weights in the
+        # checkpoint's own MXFP4 form (config 5's value distribution) instead of
+        # config 2's bf16 matrices.  The arithmetic is the same bf16 MFMA with
+        # fp32 accumulation; the weights arrive as 0.53 bytes each.
+        s4, st4, _, med4, _ = run_leg(shape, 100, 20, mxfp4=True)
+        tg, td = st4["gate_up"] * 1e-3, st4["down"] * 1e-3
+        result["prefill_mxfp4"] = {
+            "workload": f"{T} tokens, {E} experts, MXFP4 expert weights (c2's batch, c5's weights)",
+            "tokens_per_s": T / s4, "us_per_step": s4 * 1e6, "median_us_per_step": med4 * 1e6,
+            "stage_us": {k: v * 1e3 for k, v in st4.items()},
+            "gate_up_tflops": flops_gate_up / tg / 1e12,
+            "gate_up_frac_bf16_peak": flops_gate_up / tg / 1e12 / PEAK_BF16_TFLOPS,
+            "expert_gemms_tflops": (flops_gate_up + flops_down) / (tg + td) / 1e12,
+            "expert_gemms_frac_bf16_peak": (flops_gate_up + flops_down) / (tg + td) / 1e12 / PEAK_BF16_TFLOPS}
     if not args.no_cpu_baseline and L is not None:
         result["cpu_baseline"] = cpu_baseline(shape, L)
     print(json.dumps(result))
