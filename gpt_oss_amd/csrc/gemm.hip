@@ -22,11 +22,12 @@
 //     ring by DMA (global_load_lds_dwordx4), R-1 steps ahead of the MFMAs;
 //   * the column operand is private to a wave in this layout, so it never
 //     touches LDS: it is loaded into an R-slot ring of VGPRs, R-1 steps ahead.
-// The full-height configuration runs R = 5 (4 steps x 32 KB = 128 KB in flight
-// per CU: measured against 6 and 7, a deeper ring gains nothing in the main loop
-// and costs the time its longer fill takes at the start of every tile, 0.8 % of
-// the layer at 4096 tokens); the small-batch configuration, a stream of weights
-// through two or three workgroups per CU, runs R = 7.  These loads
+// The full-height configuration runs R = 4 (3 steps x 32 KB = 96 KB in flight
+// per CU: measured against 3, 5, 6 and 7, a deeper ring gains nothing in the
+// main loop and costs the time its longer fill takes at the start of every
+// tile, 0.7 % of the layer per stage at 4096 tokens; with 3 the main loop
+// starves); the small-batch configuration, a stream of weights through two or
+// three workgroups per CU, runs R = 7.  These loads
 // complete in the order they were issued, so waiting for "all but the newest n"
 // (s_waitcnt vmcnt(n)) picks out exactly the step that is needed next and
 // leaves the later ones in flight (the scattered DMA of the GATHER variant is
@@ -592,8 +593,8 @@ __global__ __launch_bounds__(C::THREADS, C::WAVES) void grouped_gemm_kernel(
 }
 
 // 4 waves, one per SIMD, each 256 rows x 64 columns (8 x 2 accumulators = all
-// 256 accumulation registers); 256 x 256 tiles; 5 ring slots.
-using CfgGemm = GemmCfg<4, 2, 5>;
+// 256 accumulation registers); 256 x 256 tiles; 4 ring slots.
+using CfgGemm = GemmCfg<4, 2, 4>;
 static_assert(CfgGemm::RBT_MAX * kRowBlock == kTileRows && CfgGemm::TILE_NB == kGemmTileNb,
               "tile plan of dispatch_scan_kernel");
 // Batches of at most 64 tokens: no expert has more than 64 rows, every tile is
