@@ -49,8 +49,31 @@ struct PlanOut {
   int tile_cap_gate_up, tile_cap_down;
 };
 
+// The tiles of expert ee in the tile sequences of both GEMMs: tile L = (expert,
+// column tile, row tile), row tile fastest.  One wave; its lanes run over the
+// expert's tiles of both GEMMs in one sweep.
+__device__ __forceinline__ void write_expert_tiles(int ee, int nmt, int rbe, int exe, int rowblk, int first,
+                                                   int lane, int n_ct_gate_up, int n_ct_down,
+                                                   const PlanOut &out) {
+  if (nmt == 0) return;
+  const int n_up = nmt * n_ct_gate_up, n = n_up + nmt * n_ct_down;
+  for (int ii = lane; ii < n; ii += 64) {
+    const bool g = ii >= n_up;
+    const int i = g ? ii - n_up : ii;
+    const int L = first * (g ? n_ct_down : n_ct_gate_up) + i;
+    const int nt = i / nmt;
+    const int mt = i - nt * nmt;
+    TileDesc d;
+    d.e = ee;
+    d.nt = nt;
+    d.rbt = rbe + (mt < exe ? 1 : 0);
+    d.rb0 = rowblk + mt * rbe + min(mt, exe);
+    if (L < (g ? out.tile_cap_down : out.tile_cap_gate_up)) (g ? out.tiles_down : out.tiles_gate_up)[L] = d;
+  }
+}
+
 __device__ __forceinline__ int build_plan(int count, int E, int n_ct_gate_up, int n_ct_down,
-                                          const PlanOut &out, int *ex_count_out,
+                                          const PlanOut &out, bool with_tiles, int *ex_count_out,
                                           int *tot_count_out = nullptr) {
   __shared__ int sh_wave[4][4];  // [wave][quantity]: the waves' sums
   __shared__ int sh_nmt[256], sh_rb[256], sh_extra[256], sh_rowblk[256];
@@ -162,29 +185,12 @@ __device__ __forceinline__ int build_plan(int count, int E, int n_ct_gate_up, in
     }
     sh_bound[g][x] = bound;
   }
-  // The tile sequences: tile L = (expert, column tile, row tile), row tile
-  // fastest.  The waves take the experts in turn, the lanes the expert's tiles.
-  for (int ee = w; ee < E; ee += 4) {
-    const int nmt = sh_nmt[ee];
-    if (nmt == 0) continue;
-    const int rbe = sh_rb[ee], exe = sh_extra[ee], rowblk = sh_rowblk[ee], first = sh_tiles[ee];
-    for (int g = 0; g < 2; g++) {
-      const int n_ct = g ? n_ct_down : n_ct_gate_up;
-      TileDesc *tiles = g ? out.tiles_down : out.tiles_gate_up;
-      const int cap = g ? out.tile_cap_down : out.tile_cap_gate_up;
-      const int n = nmt * n_ct;
-      for (int i = lane; i < n; i += 64) {
-        const int L = first * n_ct + i;
-        const int nt = i / nmt;
-        const int mt = i - nt * nmt;
-        TileDesc d;
-        d.e = ee;
-        d.nt = nt;
-        d.rbt = rbe + (mt < exe ? 1 : 0);
-        d.rb0 = rowblk + mt * rbe + min(mt, exe);
-        if (L < cap) tiles[L] = d;
-      }
-    }
+  // The tile sequences (three-launch form: written by the scatter kernel's
+  // workgroups instead, which are many).  The waves take the experts in turn.
+  if (with_tiles) {
+    for (int ee = w; ee < E; ee += 4)
+      write_expert_tiles(ee, sh_nmt[ee], sh_rb[ee], sh_extra[ee], sh_rowblk[ee], sh_tiles[ee], lane,
+                         n_ct_gate_up, n_ct_down, out);
   }
   __syncthreads();
   // keep every range within what the launch grid provides for (xcd_tile_cap)
@@ -238,7 +244,7 @@ __global__ __launch_bounds__(256) void dispatch_scan_kernel(int *__restrict__ bl
     }
   }
   int ex_count;
-  build_plan(count, E, n_ct_gate_up, n_ct_down, out, &ex_count);
+  build_plan(count, E, n_ct_gate_up, n_ct_down, out, /*with_tiles=*/false, &ex_count);
 }
 
 // Ranks inside one wave: for each of the lane's kTopK expert ids, how many of
@@ -292,11 +298,19 @@ __global__ __launch_bounds__(kDispThreads) void dispatch_scatter_kernel(
     const int *__restrict__ topk_i, const int *__restrict__ pos, int T, int E,
     const int *__restrict__ blk_base, const int *__restrict__ offsets,
     const ExpertInfo *__restrict__ info, int *__restrict__ perm, int *__restrict__ rowmap,
-    int *__restrict__ inv) {
+    int *__restrict__ inv, int n_ct_gate_up, int n_ct_down, PlanOut plan) {
   __shared__ int wave_cnt[kDispThreads / 64][256];
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int w = tid >> 6;
+  // The tile sequences of the GEMMs, from the per-expert records of the scan
+  // kernel: the waves of all workgroups take the experts in turn (in the one
+  // workgroup of the scan kernel this took as long as everything else in it).
+  for (int ee = blockIdx.x * (kDispThreads / 64) + w; ee < E; ee += gridDim.x * (kDispThreads / 64)) {
+    const ExpertInfo inf = info[ee];
+    write_expert_tiles(ee, inf.n_mt, inf.rb, inf.extra, inf.row0 / kRowBlock, inf.tile_base, lane,
+                       n_ct_gate_up, n_ct_down, plan);
+  }
   const int t = blockIdx.x * kDispThreads + tid;
   int id[kTopK] = {-1, -1, -1, -1};
   if (t < T && !(pos && pos[t] < 0)) {
@@ -378,7 +392,7 @@ __global__ __launch_bounds__(kDispThreads) void dispatch_small_kernel(
     count += c;
   }
   int ex_count, tot_count;
-  const int row0 = build_plan(tid < E ? count : 0, E, n_ct_gate_up, n_ct_down, out, &ex_count, &tot_count);
+  const int row0 = build_plan(tid < E ? count : 0, E, n_ct_gate_up, n_ct_down, out, /*with_tiles=*/true, &ex_count, &tot_count);
   sh_off[tid] = ex_count;
   sh_row0[tid] = row0;
   // -1 where the scatter below writes nothing: the padding rows of the experts
@@ -526,7 +540,8 @@ hipError_t launch_dispatch(const int *topk_i, const int *pos, int T, int E, int 
                                                        fill_rows, d.perm);
   dispatch_scan_kernel<<<1, 256, 0, s>>>(d.blk_counts, n_blk, E, n_ct_gate_up, n_ct_down, plan);
   dispatch_scatter_kernel<<<n_blk, kDispThreads, 0, s>>>(topk_i, pos, T, E, d.blk_counts, d.offsets,
-                                                         d.info, d.perm, d.rowmap, d.inv);
+                                                         d.info, d.perm, d.rowmap, d.inv, n_ct_gate_up,
+                                                         n_ct_down, plan);
   return hipGetLastError();
 }
 
