@@ -15,7 +15,7 @@ import numpy as np
 PKG = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(PKG, "libmi355_moe.so")
 
-STAGES = ["router", "dispatch", "gather", "gate_up", "down", "combine"]
+STAGES = ["router", "dispatch", "gate_up", "down", "combine"]
 
 # every symbol include/moe_abi.h declares
 SYMBOLS = [

@@ -436,35 +436,6 @@ __global__ __launch_bounds__(kDispThreads) void dispatch_small_kernel(
   }
 }
 
-// Copies the routed rows of x into the padded per-expert row space, already in
-// the A-operand fragment order of v_mfma_f32_32x32x16_bf16: fragment
-// (row block rb, k block kb) is 64 lanes x 16 bytes, lane l = row rb*32 + l%32,
-// k = 16*kb + 8*(l/32) .. +7.  Padding rows are zero.  One wave writes four
-// consecutive k blocks (4 KB) of one row block.
-constexpr int kGatherGridY = 32768;
-__global__ __launch_bounds__(256) void gather_rows_kernel(const uint16_t *__restrict__ x,
-                                                         const int *__restrict__ rowmap,
-                                                         const int *__restrict__ totals,
-                                                         uint4 *__restrict__ xg, int H) {
-  // row blocks run over the y and z dimensions of the grid (32768 each): room for
-  // any batch the handle accepts, with the k groups of a row block next to each other
-  const int rb = blockIdx.y + blockIdx.z * kGatherGridY;
-  if (rb * kRowBlock >= totals[1]) return;
-  const int lane = threadIdx.x & 63;
-  const int grp = blockIdx.x * 4 + (threadIdx.x >> 6);
-  const int kb_total = H / kFragK;
-  if (grp * 4 >= kb_total) return;
-  const int a = rowmap[rb * kRowBlock + (lane & 31)];
-  const uint16_t *src = a >= 0 ? x + (size_t)(a / kTopK) * H + grp * 64 + 8 * (lane >> 5) : nullptr;
-  uint4 *dst = xg + ((size_t)rb * kb_total + grp * 4) * 64 + lane;
-#pragma unroll
-  for (int kk = 0; kk < 4; kk++) {
-    uint4 v = make_uint4(0, 0, 0, 0);
-    if (src) v = *reinterpret_cast<const uint4 *>(src + kk * kFragK);
-    dst[kk * 64] = v;
-  }
-}
-
 // out[t,:] (+)= sum_k topk_v[t,k] * y[inv[t,k],:], slots added in order 0..3
 // (descending router score, as reduce_mlp2_slots_kernel does,
 // utility/utility.cpp:701-726).  Every token owns its K rows of y, so there
@@ -542,15 +513,6 @@ hipError_t launch_dispatch(const int *topk_i, const int *pos, int T, int E, int 
   dispatch_scatter_kernel<<<n_blk, kDispThreads, 0, s>>>(topk_i, pos, T, E, d.blk_counts, d.offsets,
                                                          d.info, d.perm, d.rowmap, d.inv, n_ct_gate_up,
                                                          n_ct_down, plan);
-  return hipGetLastError();
-}
-
-hipError_t launch_gather(const uint16_t *x, const DispatchBuffers &d, uint16_t *xg, int T, int H,
-                         int rb_cap, hipStream_t s) {
-  (void)T;
-  const int groups = H / 64;
-  dim3 grid((groups + 3) / 4, rb_cap < kGatherGridY ? rb_cap : kGatherGridY, (rb_cap + kGatherGridY - 1) / kGatherGridY);
-  gather_rows_kernel<<<grid, 256, 0, s>>>(x, d.rowmap, d.totals, reinterpret_cast<uint4 *>(xg), H);
   return hipGetLastError();
 }
 

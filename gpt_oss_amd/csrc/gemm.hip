@@ -4,10 +4,13 @@
 // (utility/utility.cpp:1108-1125; formula of run.cpp:709-726) and
 // mlp2_kernel_noatomic / mlp2_120b_kernel (matmul/matmul.cpp:1470-1914).
 //
-// Data layout.  Both operands arrive as ready-made MFMA fragments of 1 KB
-// (64 lanes x 8 bf16, see pack.hip and gather_rows_kernel), ordered
-// [row block of 32][k block of 16]: every global load is a contiguous 16
-// bytes per lane and is already in register order.
+// Data layout.  The weights and the activation between the two GEMMs are kept
+// as ready-made MFMA fragments of 1 KB (64 lanes x 8 bf16, see pack.hip and the
+// gate_up epilogue), ordered [row block of 32][k block of 16]: every global load
+// is a contiguous 16 bytes per lane and is already in register order.  The row
+// operand of gate_up is the token rows themselves, bf16 row-major, found through
+// the dispatch's row map: there is no gathered copy (gemm_tile_gl for the large
+// batches, the GATHER form of gemm_tile for the small ones).
 //
 // Tiling.  A workgroup of NW waves owns a tile of (RBT*32) rows x
 // (NW*NBW*32) columns of one expert.  The waves split the columns only: each
@@ -30,10 +33,8 @@
 // three workgroups per CU, runs R = 7.  These loads
 // complete in the order they were issued, so waiting for "all but the newest n"
 // (s_waitcnt vmcnt(n)) picks out exactly the step that is needed next and
-// leaves the later ones in flight (the scattered DMA of the GATHER variant is
-// the exception, see there).
-// Measured in the steady loop: 1113 clocks per step of 1024 MFMA clocks (tile of
-// 8 row blocks), the same in every group of every tile.
+// leaves the later ones in flight (the GATHER variant of gemm_tile counts
+// differently, see there).
 //
 // Tile order.  Workgroup ids are dealt round-robin to the 8 XCDs, each with
 // its own L2.  Logical tile ids are laid out (expert, column tile, row tile)
@@ -131,6 +132,53 @@ __device__ __forceinline__ void lds_barrier() {
   asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 }
 
+// Epilogue of the gate_up GEMM: SwiGLU of the (gate, up) accumulator pairs, bf16,
+// stored in the fragment order the down GEMM reads as its row operand.
+template <int RBT, int RS, typename C>
+__device__ __forceinline__ void gate_up_epilogue(const f32x16 (&acc)[RBT][C::NBW], void *__restrict__ outp,
+                                                 int out_ld, float limit, int rb0, int rbt, int nb0,
+                                                 int nb_valid, int cw, int rg, int lane) {
+  constexpr int NBW = C::NBW;
+  // Column blocks come in (gate, up) pairs (see pack_weight_kernel): blocks 2P
+  // and 2P+1 of the product hold gate_j and up_j of j = 32P .. 32P+31 in the
+  // same lane and register.  The activation goes out as bf16 in the fragment
+  // order the down GEMM reads as its row operand: column j is k block j/16,
+  // lane ((j%16)/8)*32 + token, element j % 8.  Registers 4g .. 4g+3 of lane
+  // (token t, half h) are j = 8g + 4h .. +3: elements 4h .. 4h+3 of the
+  // fragment lane (g % 2)*32 + t of k block g / 2.  One exchange between the
+  // lane halves (v_permlane32_swap) per dword completes the 16 bytes of every
+  // fragment lane; nothing goes through LDS.
+  uint4 *act = reinterpret_cast<uint4 *>(outp);
+  const int kb2_total = out_ld / kFragK;
+  const int P0 = (nb0 + cw * NBW) >> 1;                // first pair of this wave
+  const int pairs_valid = (nb_valid - cw * NBW) >> 1;  // >= 1 here
+#pragma unroll
+  for (int i = 0; i < RBT; i++) {
+    const int blk = i * RS + rg;
+    if (RS > 1 && blk >= rbt) break;
+#pragma unroll
+    for (int p = 0; p < NBW / 2; p++) {
+      uint32_t pk[4][2];
+#pragma unroll
+      for (int g = 0; g < 4; g++)
+#pragma unroll
+        for (int d = 0; d < 2; d++)
+          pk[g][d] = pack_bf16(
+              swiglu_shifted(acc[i][2 * p][4 * g + 2 * d], acc[i][2 * p + 1][4 * g + 2 * d], limit),
+              swiglu_shifted(acc[i][2 * p][4 * g + 2 * d + 1], acc[i][2 * p + 1][4 * g + 2 * d + 1],
+                             limit));
+      uint4 *dst = act + ((size_t)(rb0 + blk) * kb2_total + 2 * (P0 + p)) * 64 + lane;
+#pragma unroll
+      for (int kb = 0; kb < 2; kb++) {
+        // upper lane half of registers 8kb .. 8kb+3 <-> lower lane half of 8kb+4 .. 8kb+7
+        const u32x2 s0 = __builtin_amdgcn_permlane32_swap(pk[2 * kb][0], pk[2 * kb + 1][0], false, false);
+        const u32x2 s1 = __builtin_amdgcn_permlane32_swap(pk[2 * kb][1], pk[2 * kb + 1][1], false, false);
+        if (p < pairs_valid) dst[kb * 64] = make_uint4(s0[0], s1[0], s0[1], s1[1]);
+      }
+    }
+  }
+}
+
 template <int R>
 struct StageRing {
   uint4 *p[R];
@@ -168,15 +216,13 @@ struct GemmCfg {
 // wave, RBT * RS are staged per step (blocks past the tile's rbt repeat its
 // last one and are not stored).
 //
-// GATHER (gate_up of the small-batch configuration): there is no gathered copy
-// of the routed rows; the row operand's DMA reads the token rows themselves,
-// every lane at the address of its own row (rowmap) -- 32 bytes per row and
-// instruction instead of 1 KB in one piece.  That costs the main loop of a
-// large batch more than the gather kernel it saves (+25 % at 4096 tokens), but
-// when the GEMM is a stream of weights it is free and saves a launch and the
-// copy (-7 % per layer call at 64 tokens).  Such a DMA can complete after
-// register loads issued behind it, so here the waits count DMA only (see
-// WAIT_DMA_*).
+// GATHER (gate_up of the small-batch configuration): the row operand's DMA reads
+// the token rows themselves, every lane at the address of its own row (rowmap)
+// -- 32 bytes per row and instruction instead of 1 KB in one piece.  While the
+// GEMM is a stream of weights that is free; on tiles 4 to 8 row blocks high the
+// address work of 32 cache lines per instruction costs the main loop a quarter,
+// which is why the large batches fetch whole lines (gemm_tile_gl).  Here the
+// waits count DMA only (see WAIT_DMA_*).
 template <int RBT, int RS, typename C, bool GATE_UP, bool FP4, bool GATHER>
 __device__ __forceinline__ void gemm_tile(const uint4 *__restrict__ a_frag,  // [rb][KB][64]; GATHER: token rows [T][KB*2]
                                           const uint4 *__restrict__ b_frag,  // expert: [nb][KB][64], FP4: [nb/2][KB/2][64]
@@ -346,12 +392,13 @@ __device__ __forceinline__ void gemm_tile(const uint4 *__restrict__ a_frag,  // 
   // "Step s of the row operand has landed" as a bound on the vector-memory
   // counter.  The loads are issued in the order A(0) B(0) A(1) B(1) ... and
   // complete in that order, so all but the newest n outstanding means step s has
-  // landed with n = everything issued behind it.  A scattered DMA (GATHER) was
-  // seen to complete after register loads issued behind it (whole tiles of
-  // wrong rows, run to run); there the bound counts the DMAs behind step s
-  // only, which holds whatever the register loads do and waits for some of them
-  // needlessly (free while the tile is a stream of weights, +30 % on tiles of
-  // 4 to 8 row blocks, which is why GATHER stays with the small batches).
+  // landed with n = everything issued behind it.  With the scattered DMA of the
+  // GATHER form and the mixed count, wrong token rows were once seen in this
+  // configuration (several workgroups per CU, ring of 7), different from run to
+  // run; the cause was never established (the same scattered DMA with the mixed
+  // count gives the same bits in every run on the large batches).  Here the
+  // bound counts the DMAs behind step s only, which holds whatever the register
+  // loads do and costs nothing while the tile is a stream of weights.
   constexpr int WAIT_DMA_FILL = GATHER ? LA * (R - 1) : LPS * (R - 2) + LA;  // A(0), A(0..R-1) issued
   constexpr int WAIT_DMA_STEP = GATHER ? LA * (R - 2) : LPS * (R - 2);       // A(ks+1) at step ks
 
@@ -460,44 +507,7 @@ __device__ __forceinline__ void gemm_tile(const uint4 *__restrict__ a_frag,  // 
   // Epilogue.
   if (cw * NBW >= nb_valid) return;  // a wave without columns (last column tile only)
   if (GATE_UP) {
-    // Column blocks come in (gate, up) pairs (see pack_weight_kernel): blocks 2P
-    // and 2P+1 of the product hold gate_j and up_j of j = 32P .. 32P+31 in the
-    // same lane and register.  The activation goes out as bf16 in the fragment
-    // order the down GEMM reads as its row operand: column j is k block j/16,
-    // lane ((j%16)/8)*32 + token, element j % 8.  Registers 4g .. 4g+3 of lane
-    // (token t, half h) are j = 8g + 4h .. +3: elements 4h .. 4h+3 of the
-    // fragment lane (g % 2)*32 + t of k block g / 2.  One exchange between the
-    // lane halves (v_permlane32_swap) per dword completes the 16 bytes of every
-    // fragment lane; nothing goes through LDS.
-    uint4 *act = reinterpret_cast<uint4 *>(outp);
-    const int kb2_total = out_ld / kFragK;
-    const int P0 = (nb0 + cw * NBW) >> 1;                // first pair of this wave
-    const int pairs_valid = (nb_valid - cw * NBW) >> 1;  // >= 1 here
-#pragma unroll
-    for (int i = 0; i < RBT; i++) {
-      const int blk = i * RS + rg;
-      if (RS > 1 && blk >= rbt) break;
-#pragma unroll
-      for (int p = 0; p < NBW / 2; p++) {
-        uint32_t pk[4][2];
-#pragma unroll
-        for (int g = 0; g < 4; g++)
-#pragma unroll
-          for (int d = 0; d < 2; d++)
-            pk[g][d] = pack_bf16(
-                swiglu_shifted(acc[i][2 * p][4 * g + 2 * d], acc[i][2 * p + 1][4 * g + 2 * d], limit),
-                swiglu_shifted(acc[i][2 * p][4 * g + 2 * d + 1], acc[i][2 * p + 1][4 * g + 2 * d + 1],
-                               limit));
-        uint4 *dst = act + ((size_t)(rb0 + blk) * kb2_total + 2 * (P0 + p)) * 64 + lane;
-#pragma unroll
-        for (int kb = 0; kb < 2; kb++) {
-          // upper lane half of registers 8kb .. 8kb+3 <-> lower lane half of 8kb+4 .. 8kb+7
-          const u32x2 s0 = __builtin_amdgcn_permlane32_swap(pk[2 * kb][0], pk[2 * kb + 1][0], false, false);
-          const u32x2 s1 = __builtin_amdgcn_permlane32_swap(pk[2 * kb][1], pk[2 * kb + 1][1], false, false);
-          if (p < pairs_valid) dst[kb * 64] = make_uint4(s0[0], s1[0], s0[1], s1[1]);
-        }
-      }
-    }
+    gate_up_epilogue<RBT, RS, C>(acc, outp, out_ld, limit, rb0, rbt, nb0, nb_valid, cw, rg, lane);
   } else {
     constexpr int LD = C::EPI_LD;  // +8 floats keep the two lane halves on different banks
     float *y = reinterpret_cast<float *>(outp);
@@ -530,6 +540,278 @@ __device__ __forceinline__ void gemm_tile(const uint4 *__restrict__ a_frag,  // 
   }
 }
 
+// double stages of the row operand in gemm_tile_gl (3: 96 KB of LDS, 4: 128 KB)
+constexpr int kLineStages = 4;
+
+// gate_up of the large batches without a gathered copy of the routed rows: the
+// row operand's DMA reads the token rows themselves, WHOLE CACHE LINES at a time.
+// One instruction fetches 8 rows x 128 bytes (64 k); a scattered DMA that takes
+// 32 bytes of 32 rows per instruction (the small-batch form in gemm_tile) costs
+// the main loop a quarter more, and 64 bytes of 16 rows an eighth.
+//
+// So the row operand is staged in double steps: a double stage holds 64 k of
+// all rows of the tile (two 16 KB arrays: row blocks 0-3 and 4-7), R2 of them
+// form the ring, and the refill comes every other step.  Wave w fetches rows
+// 8w .. 8w+7 of every row block; inside its kilobyte a lane holds one 16-byte
+// piece of one of the 8 rows, and WHICH is chosen so that (a) the four lanes of
+// a quad read 64 contiguous bytes of one row and (b) the MFMA operand reads
+// (lane = row, all lanes the same piece) find 8 consecutive rows on the 8
+// different 16-byte slots of 128 bytes of LDS and 16 consecutive rows on the 16
+// of 256 bytes: quad Q = 4 * (row / 2) + 2 * (half of the line ^ w % 2) + row % 2,
+// and lane j of the quad holds piece (j - row / 2) mod 4 of that half.
+//
+// The column operand keeps its ring of RB register slots of one step each.
+// Loads are issued in the order  A2(0) A2(1) B(0) A2(2) B(1) B(2) A2(3) | step 0:
+// B(3) | step 1: B(4) A2(4) | step 2: B(5) | step 3: B(6) A2(5) | ...  (R2 = RB =
+// 4).  The counted wait in the middle of a step leaves the newest 2 LB + LA2
+// loads in flight (see gemm_tile for the assumption): that covers A2(d+1), which
+// an odd step 2d+1 needs, and B(ks+1), which every step's successor needs.  Even
+// steps need no barrier: they read a double stage that landed before the
+// previous odd step's barrier and refill nothing.
+template <int RBT, int RS, typename C, bool FP4>
+__device__ __forceinline__ void gemm_tile_gl(const uint4 *__restrict__ x_rows,  // token rows [T][KB * 2] of 16 bytes
+                                             const uint4 *__restrict__ b_frag,
+                                             const uint16_t *__restrict__ b_scale, int KB, int rb0, int rbt,
+                                             int nb0, int nb_valid, const int *__restrict__ rowmap,
+                                             const float *__restrict__ bias_a,
+                                             const float *__restrict__ bias_b, void *__restrict__ outp,
+                                             int out_ld, float limit, uint4 *__restrict__ s0,
+                                             uint4 *__restrict__ s1, uint4 *__restrict__ s2,
+                                             uint4 *__restrict__ s3, uint4 *__restrict__ s4,
+                                             uint4 *__restrict__ s5, uint4 *__restrict__ s6,
+                                             uint4 *__restrict__ s7) {
+  constexpr int NBW = C::NBW, KPS = C::KPS, RB = C::R, NW = C::NW, R2 = kLineStages;
+  static_assert(KPS == 2 && NW == 4 && RB == 4 && C::RBT_MAX == 8 && (RS == 1 || RS == 2), "shape of the line gather");
+  constexpr int NB = RBT * RS;                // row blocks staged per step
+  constexpr int LA2 = NB;                     // DMA loads per wave and double step: one per row block
+  constexpr int LB = FP4 ? 2 : NBW * KPS;     // register loads per wave and step
+  static_assert(!FP4 || NBW == 2, "an MXFP4 chunk holds the pair of column blocks of one wave");
+  constexpr int NM = RBT * NBW;               // MFMAs per k block
+  constexpr int DEC = FP4 ? NBW : 0;
+  static_assert(R2 == 3 || R2 == 4, "first fillings written out below; with 2 an odd step would have to wait for 2 * LB");
+  constexpr int WAIT_FILL = R2 == 4 ? 3 * LB + 3 * LA2 : 3 * LB + 2 * LA2;  // the loads behind A2(0) in the first filling
+  constexpr int WAIT_MID = 2 * LB + LA2;                                     // see the steps
+  static_assert(WAIT_FILL <= 63 && WAIT_MID <= 63, "vmcnt is a 6-bit counter");
+  uint4 *const arr[8] = {s0, s1, s2, s3, s4, s5, s6, s7};
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int cw = RS == 1 ? w : w % (NW / RS);
+  const int rg = RS == 1 ? 0 : w / (NW / RS);
+
+  float4 bias_g[NBW / 2][4], bias_u[NBW / 2][4];
+  {
+    const int P_last = ((nb0 + nb_valid) >> 1) - 1;
+    const int P0 = (nb0 + cw * NBW) >> 1;
+#pragma unroll
+    for (int p = 0; p < NBW / 2; p++) {
+      const int P = min(P0 + p, P_last);
+#pragma unroll
+      for (int g = 0; g < 4; g++) {
+        const int j = kRowBlock * P + 8 * g + 4 * (lane >> 5);
+        bias_g[p][g] = *reinterpret_cast<const float4 *>(bias_a + j);
+        bias_u[p][g] = *reinterpret_cast<const float4 *>(bias_b + j);
+      }
+    }
+  }
+  f32x16 acc[RBT][NBW];
+  const int n_steps = KB / KPS;  // even: the depth is a multiple of 64
+  const int last = n_steps - 1, last_d = n_steps / 2 - 1;
+
+  // this lane's source in a double step of row block m: its token's row and its piece of the line
+  uint32_t lane_src[LA2];
+  {
+    const int Q = lane >> 2, j = lane & 3;  // quad Q of the kilobyte: row 2 * (Q / 4) + Q % 2, one half of its line
+    const int row8 = 2 * (Q >> 2) + (Q & 1);
+    const int piece = 4 * (((Q >> 1) & 1) ^ (w & 1)) + ((j - (Q >> 2)) & 3);
+#pragma unroll
+    for (int m = 0; m < LA2; m++) {
+      const int blk = RS == 1 ? m : min(m, rbt - 1);
+      const int a = rowmap[(rb0 + blk) * kRowBlock + 8 * w + row8];
+      const int tok = a >= 0 ? a / kTopK : 0;  // padding rows read token 0; their products are never used
+      lane_src[m] = (uint32_t)tok * (uint32_t)(KB * 2) + piece;
+    }
+  }
+  // where this lane finds its operand of (parity of the step, k block) inside a row block's 4 KB
+  int lane_rd[2][KPS];
+  {
+    const int r = lane & 31, h = lane >> 5, sub = r >> 3, row8 = r & 7;
+#pragma unroll
+    for (int par = 0; par < 2; par++)
+#pragma unroll
+      for (int kk = 0; kk < KPS; kk++)
+        lane_rd[par][kk] = sub * 64 + (4 * (row8 >> 1) + 2 * (par ^ (sub & 1)) + (row8 & 1)) * 4 +
+                           ((kk * 2 + h + (row8 >> 1)) & 3);
+  }
+  const uint4 *b_src[NBW];
+  const uint16_t *s_src = nullptr;
+  if (FP4) {
+    const size_t pair = (size_t)((nb0 + min(cw * NBW, nb_valid - NBW)) >> 1);
+    b_src[0] = b_frag + pair * n_steps * 64 + lane;
+    s_src = b_scale + pair * n_steps * 32 + (lane & 31);
+  } else {
+#pragma unroll
+    for (int j = 0; j < NBW; j++)
+      b_src[j] = b_frag + (size_t)(nb0 + min(cw * NBW + j, nb_valid - 1)) * KB * 64 + lane;
+  }
+
+  // double step jd of row block m into double stage slot d
+  auto issue_a2 = [&](int d, int jd, int m) {
+    dma_to_lds_16(x_rows + lane_src[m] + jd * 8, arr[2 * d + (m >= 4 ? 1 : 0)] + ((m & 3) * 4 + w) * 64);
+  };
+  u32x4 bq[RB][FP4 ? 1 : LB];
+  uint32_t bsc[RB];
+  auto issue_b = [&](int slot, int ks, int m) {
+    if (FP4) {
+      if (m == 0) {
+        bq[slot][0] = *reinterpret_cast<const u32x4 *>(b_src[0] + (size_t)ks * 64);
+      } else {
+        bsc[slot] = s_src[(size_t)ks * 32];
+      }
+    } else {
+      bq[slot][m] = *reinterpret_cast<const u32x4 *>(b_src[m / KPS] + (size_t)(ks * KPS + m % KPS) * 64);
+    }
+  };
+  bf16x8 bdec[NBW][KPS];
+  auto decode = [&](int slot, int j, int kk) {
+    const float scale = __uint_as_float(((bsc[slot] >> (8 * j)) & 0xffu) << 23);
+    const uint32_t nib = bq[slot][0][j * KPS + kk];
+    const bf16x2 p0 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(nib, scale, 0);
+    const bf16x2 p1 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(nib, scale, 1);
+    const bf16x2 p2 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(nib, scale, 2);
+    const bf16x2 p3 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(nib, scale, 3);
+    bdec[j][kk] = bf16x8{p0[0], p0[1], p1[0], p1[1], p2[0], p2[1], p3[0], p3[1]};
+  };
+  bf16x8 fa[2][RBT];
+  // fragment of the wave's row block i from double stage slot d
+  auto read_a = [&](int d, int par, int kk, int buf, int i) {
+    const uint4 *st = arr[2 * d + (i * RS >= 4 ? 1 : 0)];
+    fa[buf][i] = __builtin_bit_cast(bf16x8, st[(((i * RS + rg) & 3) * 4) * 64 + lane_rd[par][kk]]);
+  };
+  auto mma = [](bf16x8 rows, bf16x8 colv, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(colv, rows, c, 0, 0, 0);
+  };
+  auto cols_of = [&](int slot, int j, int kk) {
+    if constexpr (FP4) {
+      return bdec[j][kk];
+    } else {
+      return __builtin_bit_cast(bf16x8, bq[slot][j * KPS + kk]);
+    }
+  };
+
+  // A2(0) A2(1) B(0) A2(2) B(1) B(2) A2(3)
+  auto issue_a2_all = [&](int d, int jd) {
+#pragma unroll
+    for (int m = 0; m < LA2; m++) issue_a2(d, min(jd, last_d), m);
+  };
+  auto issue_b_all = [&](int slot, int ks) {
+#pragma unroll
+    for (int m = 0; m < LB; m++) issue_b(slot, min(ks, last), m);
+  };
+  if constexpr (R2 == 4) {  // A2(0) A2(1) B(0) A2(2) B(1) B(2) | A2(3)
+    issue_a2_all(0, 0);
+    issue_a2_all(1, 1);
+    __builtin_amdgcn_sched_barrier(0);  // the counted waits rely on this issue order
+    issue_b_all(0, 0);
+    issue_a2_all(2, 2);
+  } else {  // A2(0) B(0) A2(1) B(1) B(2) | A2(2)
+    issue_a2_all(0, 0);
+    __builtin_amdgcn_sched_barrier(0);
+    issue_b_all(0, 0);
+    issue_a2_all(1, 1);
+  }
+  __builtin_amdgcn_sched_barrier(0);
+  issue_b_all(1, 1);
+  issue_b_all(2, 2);
+  __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+  for (int p = 0; p < NBW / 2; p++)
+#pragma unroll
+    for (int g = 0; g < 4; g++)
+#pragma unroll
+      for (int i = 0; i < RBT; i++) {
+        const float4 bg = bias_g[p][g], bu = bias_u[p][g];
+        acc[i][2 * p][4 * g + 0] = bg.x; acc[i][2 * p][4 * g + 1] = bg.y;
+        acc[i][2 * p][4 * g + 2] = bg.z; acc[i][2 * p][4 * g + 3] = bg.w;
+        acc[i][2 * p + 1][4 * g + 0] = bu.x + 1.0f; acc[i][2 * p + 1][4 * g + 1] = bu.y + 1.0f;
+        acc[i][2 * p + 1][4 * g + 2] = bu.z + 1.0f; acc[i][2 * p + 1][4 * g + 3] = bu.w + 1.0f;
+      }
+  issue_a2_all(R2 - 1, R2 - 1);
+  WAIT_VMCNT(WAIT_FILL);
+  lds_barrier();
+#pragma unroll
+  for (int i = 0; i < RBT; i++) read_a(0, 0, 0, 0, i);
+  if (FP4) {
+#pragma unroll
+    for (int j = 0; j < NBW; j++) decode(0, j, 0);
+  }
+
+  // Step ks = 2 jd + par, u = ks mod PERIOD: column slot u % RB, double stage (u / 2) % R2.
+  auto step = [&](auto u_c, int ks) {
+    constexpr int u = decltype(u_c)::value;
+    constexpr int slot = u % RB, d = (u / 2) % R2, par = u % 2;
+    constexpr int LAX = par ? LA2 : 0;             // the refill comes with the odd steps
+    constexpr int dn = par ? (d + 1) % R2 : d;     // the next step's double stage
+    constexpr int SIDE1 = (RBT + LB + DEC + NM - 1) / NM;
+    constexpr int SIDE2 = (LAX + RBT + DEC + NM - 1) / NM;
+    const int ks_b = min(ks + RB - 1, last);
+    const int jd_a = min(ks / 2 + R2, last_d);
+#pragma unroll
+    for (int m = 0; m < NM; m++) {
+#pragma unroll
+      for (int t = m * SIDE1; t < (m + 1) * SIDE1; t++) {
+        if (t < RBT) {
+          read_a(d, par, 1, 1, t);
+        } else if (t < RBT + LB) {
+          issue_b((slot + RB - 1) % RB, ks_b, t - RBT);
+        } else if (t < RBT + LB + DEC) {
+          decode(slot, t - RBT - LB, 1);
+        }
+      }
+      acc[m / NBW][m % NBW] = mma(fa[0][m / NBW], cols_of(slot, m % NBW, 0), acc[m / NBW][m % NBW]);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    // Every step says in its middle what has landed, as a count: all but the
+    // column loads of the last two steps and the double step issued between
+    // them.  An odd step needs A2(jd+1), which lies further back, for the
+    // fragment reads that follow; every step needs B(ks+1) for its successor's
+    // first MFMA, and with the count given here the compiler adds no wait of its
+    // own (left to itself it waits for ALL loads before some of the steps).
+    WAIT_VMCNT(WAIT_MID);
+    if constexpr (par == 1) {
+      lds_barrier();  // double step jd+1 is complete in LDS; every wave is done with double stage d
+    } else {
+      __builtin_amdgcn_sched_barrier(0);
+    }
+#pragma unroll
+    for (int m = 0; m < NM; m++) {
+#pragma unroll
+      for (int t = m * SIDE2; t < (m + 1) * SIDE2; t++) {
+        if (t < LAX) {
+          issue_a2(d, jd_a, t);
+        } else if (t < LAX + RBT) {
+          read_a(dn, par ^ 1, 0, 0, t - LAX);
+        } else if (t < LAX + RBT + DEC) {
+          decode((slot + 1) % RB, t - LAX - RBT, 0);
+        }
+      }
+      acc[m / NBW][m % NBW] = mma(fa[1][m / NBW], cols_of(slot, m % NBW, 1), acc[m / NBW][m % NBW]);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+  constexpr int PERIOD = R2 == 3 ? 12 : 2 * R2;  // a multiple of 2 * R2 and of RB
+  static_assert(PERIOD % RB == 0 && PERIOD % (2 * R2) == 0, "one unrolled round serves both rings");
+  int ks0 = 0;
+  for (; ks0 + PERIOD <= n_steps; ks0 += PERIOD)
+    static_for<PERIOD>([&](auto u_c) { step(u_c, ks0 + decltype(u_c)::value); });
+  static_for<PERIOD - 1>([&](auto u_c) {
+    if (ks0 + decltype(u_c)::value < n_steps) step(u_c, ks0 + decltype(u_c)::value);
+  });
+
+  if (cw * NBW >= nb_valid) return;  // a wave without columns (last column tile only)
+  gate_up_epilogue<RBT, RS, C>(acc, outp, out_ld, limit, rb0, rbt, nb0, nb_valid, cw, rg, lane);
+}
+
 template <typename C, bool GATE_UP, bool FP4, bool GATHER>
 __global__ __launch_bounds__(C::THREADS, C::WAVES) void grouped_gemm_kernel(
     const uint4 *__restrict__ a_frag, const uint4 *__restrict__ w_frag,
@@ -541,7 +823,7 @@ __global__ __launch_bounds__(C::THREADS, C::WAVES) void grouped_gemm_kernel(
   constexpr int R = C::R;
   static_assert(R <= 7, "seven stage arrays are declared below");
   __shared__ uint4 st0[C::STAGE], st1[C::STAGE], st2[C::STAGE], st3[C::STAGE], st4[C::STAGE],
-      st5[C::STAGE], st6[C::STAGE];
+      st5[C::STAGE], st6[C::STAGE], st7[C::STAGE];  // those a variant does not use take no room
   __shared__ uint4 epi[C::NW * C::EPI_WAVE];
   const int KB = K / kFragK;
   const int nb_total = (GATE_UP ? 2 * N : N) / kRowBlock;  // weight row blocks per expert
@@ -555,8 +837,19 @@ __global__ __launch_bounds__(C::THREADS, C::WAVES) void grouped_gemm_kernel(
   const uint16_t *b_scale = FP4 ? w_scale + (size_t)tc.e * nb_total * KB * 8 : nullptr;
   const float *ba = bias_a + (size_t)tc.e * N;
   const float *bb = GATE_UP ? bias_b + (size_t)tc.e * N : nullptr;
-#define MOE_TILE_RS(n, rs) \
-  gemm_tile<n, rs, C, GATE_UP, FP4, GATHER>(a_frag, b_frag, b_scale, KB, tc.rb0, tc.rbt, nb0, nb_valid, rowmap, ba, bb, outp, N, limit, st0, st1, st2, st3, st4, st5, st6, epi)
+  // large batches of gate_up read the token rows by whole cache lines (gemm_tile_gl)
+  constexpr bool LINES = GATHER && C::RBT_MAX == 8;
+#define MOE_TILE_RS(n, rs)                                                                                    \
+  do {                                                                                                        \
+    if constexpr (LINES && rs <= 2) {                                                                         \
+      gemm_tile_gl<n, rs, C, FP4>(a_frag, b_frag, b_scale, KB, tc.rb0, tc.rbt, nb0, nb_valid, rowmap, ba, bb, \
+                                  outp, N, limit, st0, st1, st2, st3, st4, st5, st6, st7);                    \
+    } else {                                                                                                  \
+      gemm_tile<n, rs, C, GATE_UP, FP4, GATHER>(a_frag, b_frag, b_scale, KB, tc.rb0, tc.rbt, nb0, nb_valid,   \
+                                                rowmap, ba, bb, outp, N, limit, st0, st1, st2, st3, st4, st5, \
+                                                st6, epi);                                                    \
+    }                                                                                                         \
+  } while (0)
 #define MOE_TILE(n) MOE_TILE_RS(n, 1)
   if constexpr (C::RBT_MAX == 8) {
     // the last column tile, when only a quarter or half of the waves have columns in it
@@ -625,17 +918,17 @@ static hipError_t launch_gemm(const uint4 *a, const uint4 *w, const uint16_t *w_
   return hipGetLastError();
 }
 
-hipError_t launch_gate_up(const uint16_t *xg, const uint16_t *x, const void *w1,
-                          const uint16_t *w1_scale, const float *b1g, const float *b1u,
-                          const DispatchBuffers &d, uint16_t *act, int H, int IM, float limit, int mt_cap,
-                          int max_rows, hipStream_t s) {
-  static_assert(kSmallBatchTokens == kSmallBatchRows, "gate_up_gathers() and the small-batch configuration");
+hipError_t launch_gate_up(const uint16_t *x, const void *w1, const uint16_t *w1_scale, const float *b1g,
+                          const float *b1u, const DispatchBuffers &d, uint16_t *act, int H, int IM,
+                          float limit, int mt_cap, int max_rows, hipStream_t s) {
+  static_assert(kSmallBatchTokens == kSmallBatchRows, "small_batch() and the small-batch configuration");
   const uint4 *w = reinterpret_cast<const uint4 *>(w1);
-  if (gate_up_gathers(max_rows))
-    return launch_gemm<CfgGemmSmall, true, true>(reinterpret_cast<const uint4 *>(x), w, w1_scale, b1g, b1u,
-                                                 d, act, H, IM, limit, mt_cap, s);
-  return launch_gemm<CfgGemm, true>(reinterpret_cast<const uint4 *>(xg), w, w1_scale, b1g, b1u, d, act, H,
-                                    IM, limit, mt_cap, s);
+  const uint4 *rows = reinterpret_cast<const uint4 *>(x);
+  // either way the row operand is read from the token rows: 32 bytes of 32 rows per
+  // instruction in the small-batch configuration, whole lines of 8 rows otherwise
+  if (small_batch(max_rows))
+    return launch_gemm<CfgGemmSmall, true, true>(rows, w, w1_scale, b1g, b1u, d, act, H, IM, limit, mt_cap, s);
+  return launch_gemm<CfgGemm, true, true>(rows, w, w1_scale, b1g, b1u, d, act, H, IM, limit, mt_cap, s);
 }
 
 hipError_t launch_down(const uint16_t *act, const void *w2, const uint16_t *w2_scale, const float *b2,

@@ -66,7 +66,6 @@ struct moe_handle {
   int n_blk_cap = 0;
   int disp_tokens = -1;  // batch of the last moe_dispatch (stage-level calls), -1: none
   // expert pipeline
-  uint16_t *xg = nullptr;   // gathered rows, bf16 fragments
   uint16_t *act = nullptr;  // SwiGLU output, bf16 fragments
   float *y = nullptr;       // down output [a_pad_cap, H]
   uint16_t *t_norm = nullptr;  // normalised rows of moe_block_forward [max_tokens, H], allocated on first use
@@ -99,6 +98,9 @@ int check_forward_args(moe_handle *h, int layer, const void *x, int n_tokens, co
   if (n_tokens > h->cfg.max_tokens)
     return fail(MOE_ERR_CAPACITY, "n_tokens %d exceeds max_tokens %d", n_tokens, h->cfg.max_tokens);
   if (n_tokens > 0 && (!x || !out)) return fail(MOE_ERR_BAD_ARG, "null device pointer");
+  // the kernels read the rows of x in 16-byte pieces (a row is a multiple of 128 bytes)
+  if ((reinterpret_cast<uintptr_t>(x) & 15) != 0)
+    return fail(MOE_ERR_BAD_ARG, "x is not 16-byte aligned");
   if (!h->layers[layer].uploaded)
     return fail(MOE_ERR_STATE, "layer %d has no weights (moe_upload_layer not called)", layer);
   return MOE_OK;
@@ -131,8 +133,9 @@ inline int down_col_tiles(const moe_config &c) {
   return (c.hidden / kRowBlock + kGemmTileNb - 1) / kGemmTileNb;
 }
 
-// Stages 3-5 on the plan of the last dispatch: gather (large batches), gate_up
-// GEMM with the SwiGLU, down GEMM.  Leaves the per-assignment rows in h->y.
+// Stages 3-4 on the plan of the last dispatch: gate_up GEMM with the SwiGLU (it
+// reads the routed token rows itself, there is no gathered copy), down GEMM.
+// Leaves the per-assignment rows in h->y.
 // max_rows: no expert is given more rows than this (T when the ids of a token are distinct).
 int run_gemms(moe_handle *h, int layer, const uint16_t *x, int T, int max_rows, hipStream_t s,
               StageTimer &tm) {
@@ -140,12 +143,9 @@ int run_gemms(moe_handle *h, int layer, const uint16_t *x, int T, int max_rows, 
   const LayerWeights &lw = h->layers[layer];
   const int A = T * kTopK;
   const int mt_cap = A / kTileRows + c.experts;
-  const int rb_cap = (A + kTileGran * c.experts + kRowBlock - 1) / kRowBlock;
-  HIP_TRY(tm.mark(MOE_STAGE_GATHER));
-  if (!gate_up_gathers(max_rows)) HIP_TRY(launch_gather(x, h->disp, h->xg, T, c.hidden, rb_cap, s));
   HIP_TRY(tm.mark(MOE_STAGE_GATE_UP));
-  HIP_TRY(launch_gate_up(h->xg, x, lw.w1q ? static_cast<const void *>(lw.w1q) : lw.w1, lw.w1s, lw.b1g,
-                         lw.b1u, h->disp, h->act, c.hidden, c.inter, c.swiglu_limit, mt_cap, max_rows, s));
+  HIP_TRY(launch_gate_up(x, lw.w1q ? static_cast<const void *>(lw.w1q) : lw.w1, lw.w1s, lw.b1g, lw.b1u,
+                         h->disp, h->act, c.hidden, c.inter, c.swiglu_limit, mt_cap, max_rows, s));
   HIP_TRY(tm.mark(MOE_STAGE_DOWN));
   HIP_TRY(launch_down(h->act, lw.w2q ? static_cast<const void *>(lw.w2q) : lw.w2, lw.w2s, lw.b2,
                       h->disp, h->y, c.hidden, c.inter, mt_cap, max_rows, s));
@@ -237,7 +237,6 @@ int moe_create(const moe_config *cfg, moe_handle **out) {
   }
   ALLOC(h->disp.tiles_gate_up, (size_t)h->disp.tile_cap_gate_up);
   ALLOC(h->disp.tiles_down, (size_t)h->disp.tile_cap_down);
-  ALLOC(h->xg, (size_t)h->a_pad_cap * H);
   ALLOC(h->act, (size_t)h->a_pad_cap * IM);
   ALLOC(h->y, (size_t)h->a_pad_cap * H);
 #undef ALLOC
@@ -264,7 +263,7 @@ int moe_destroy(moe_handle *h) {
   (void)hipFree(h->disp.blk_counts); (void)hipFree(h->disp.offsets); (void)hipFree(h->disp.perm);
   (void)hipFree(h->disp.rowmap); (void)hipFree(h->disp.inv); (void)hipFree(h->disp.info); (void)hipFree(h->disp.totals);
   (void)hipFree(h->disp.tiles_gate_up); (void)hipFree(h->disp.tiles_down);
-  (void)hipFree(h->xg); (void)hipFree(h->act); (void)hipFree(h->y); (void)hipFree(h->t_norm);
+  (void)hipFree(h->act); (void)hipFree(h->y); (void)hipFree(h->t_norm);
   for (hipEvent_t ev : h->events) (void)hipEventDestroy(ev);
   delete h;
   return MOE_OK;

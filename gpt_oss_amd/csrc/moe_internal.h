@@ -131,20 +131,14 @@ struct DispatchBuffers {
 };
 hipError_t launch_dispatch(const int *topk_i, const int *pos, int T, int E, int n_ct_gate_up,
                            int n_ct_down, const DispatchBuffers &d, hipStream_t s);
-hipError_t launch_gather(const uint16_t *x, const DispatchBuffers &d, uint16_t *xg, int T, int H,
-                         int rb_cap, hipStream_t s);
-
-// w*_scale == nullptr: w* are bf16 fragments; otherwise MXFP4 chunks + scale bytes.
-// When no expert can have more than this many rows (the small-batch
-// configuration of the GEMMs) the gate_up GEMM reads the token rows itself,
-// through rowmap, and launch_gather is not needed; above, it reads the gathered
-// copy xg.
+// gate_up reads the routed token rows of x itself, through rowmap; there is no
+// gathered copy.  Batches in which no expert has more than kSmallBatchRows rows
+// run the small-batch configuration of both GEMMs.
 constexpr int kSmallBatchRows = 64;
-inline bool gate_up_gathers(int max_rows) { return max_rows <= kSmallBatchRows; }
-hipError_t launch_gate_up(const uint16_t *xg, const uint16_t *x, const void *w1,
-                          const uint16_t *w1_scale, const float *b1g, const float *b1u,
-                          const DispatchBuffers &d, uint16_t *act, int H, int IM, float limit, int mt_cap,
-                          int max_rows, hipStream_t s);
+inline bool small_batch(int max_rows) { return max_rows <= kSmallBatchRows; }
+hipError_t launch_gate_up(const uint16_t *x, const void *w1, const uint16_t *w1_scale, const float *b1g,
+                          const float *b1u, const DispatchBuffers &d, uint16_t *act, int H, int IM,
+                          float limit, int mt_cap, int max_rows, hipStream_t s);
 hipError_t launch_down(const uint16_t *act, const void *w2, const uint16_t *w2_scale, const float *b2,
                        const DispatchBuffers &d, float *y, int H, int IM, int mt_cap, int max_rows,
                        hipStream_t s);

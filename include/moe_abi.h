@@ -57,11 +57,10 @@ typedef struct {
 enum {
   MOE_STAGE_ROUTER = 0,   /* logits + bias + top-4 + softmax        */
   MOE_STAGE_DISPATCH = 1, /* histogram + scan + stable permutation  */
-  MOE_STAGE_GATHER = 2,   /* rows copied into per-expert segments   */
-  MOE_STAGE_GATE_UP = 3,  /* grouped GEMM 1 + clamped SwiGLU        */
-  MOE_STAGE_DOWN = 4,     /* grouped GEMM 2 + bias                  */
-  MOE_STAGE_COMBINE = 5,  /* weighted sum back to token order       */
-  MOE_NUM_STAGES = 6
+  MOE_STAGE_GATE_UP = 2,  /* grouped GEMM 1 + clamped SwiGLU (reads the routed token rows itself) */
+  MOE_STAGE_DOWN = 3,     /* grouped GEMM 2 + bias                  */
+  MOE_STAGE_COMBINE = 4,  /* weighted sum back to token order       */
+  MOE_NUM_STAGES = 5
 };
 
 /* Allocates weights and workspaces for cfg on the current device.

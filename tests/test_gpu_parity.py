@@ -520,6 +520,9 @@ def test_error_paths_and_profiling(c2):
     with pytest.raises(abi.MoeError) as e:
         fresh.forward(0, dx, None, 16, dout)
     assert e.value.code == -5
+    with pytest.raises(abi.MoeError) as e:  # the rows of x are read in 16-byte pieces
+        m.forward(0, dx.ptr + 2, None, 8, dout)
+    assert e.value.code == -1
     m.forward(0, dx, None, 0, dout)  # empty batch is a no-op
     m.profile_enable(3)
     for _ in range(3):
