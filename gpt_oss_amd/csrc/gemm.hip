@@ -561,7 +561,7 @@ constexpr int kLineStages = 4;
 // and lane j of the quad holds piece (j - row / 2) mod 4 of that half.
 //
 // The column operand keeps its ring of RB register slots of one step each.
-// Loads are issued in the order  A2(0) A2(1) B(0) A2(2) B(1) B(2) A2(3) | step 0:
+// Loads are issued in the order  B(0) B(1) B(2) A2(0) A2(1) A2(2) A2(3) | step 0:
 // B(3) | step 1: B(4) A2(4) | step 2: B(5) | step 3: B(6) A2(5) | ...  (R2 = RB =
 // 4).  The counted wait in the middle of a step leaves the newest 2 LB + LA2
 // loads in flight (see gemm_tile for the assumption): that covers A2(d+1), which
@@ -588,8 +588,8 @@ __device__ __forceinline__ void gemm_tile_gl(const uint4 *__restrict__ x_rows,  
   static_assert(!FP4 || NBW == 2, "an MXFP4 chunk holds the pair of column blocks of one wave");
   constexpr int NM = RBT * NBW;               // MFMAs per k block
   constexpr int DEC = FP4 ? NBW : 0;
-  static_assert(R2 == 3 || R2 == 4, "first fillings written out below; with 2 an odd step would have to wait for 2 * LB");
-  constexpr int WAIT_FILL = R2 == 4 ? 3 * LB + 3 * LA2 : 3 * LB + 2 * LA2;  // the loads behind A2(0) in the first filling
+  static_assert(R2 >= 3, "with 2 double stages an odd step would have to wait for all but 2 * LB loads");
+  constexpr int WAIT_FILL = (R2 - 1) * LA2;  // the loads behind A2(0) in the first filling
   constexpr int WAIT_MID = 2 * LB + LA2;                                     // see the steps
   static_assert(WAIT_FILL <= 63 && WAIT_MID <= 63, "vmcnt is a 6-bit counter");
   uint4 *const arr[8] = {s0, s1, s2, s3, s4, s5, s6, s7};
@@ -618,18 +618,19 @@ __device__ __forceinline__ void gemm_tile_gl(const uint4 *__restrict__ x_rows,  
   const int n_steps = KB / KPS;  // even: the depth is a multiple of 64
   const int last = n_steps - 1, last_d = n_steps / 2 - 1;
 
-  // this lane's source in a double step of row block m: its token's row and its piece of the line
+  // this lane's source in a double step of row block m: its token's row and its piece of the line.
+  // The row map is asked for here; the answer is used after the column operand's
+  // first loads have gone out (below), so that its latency costs the tile nothing.
   uint32_t lane_src[LA2];
+  int lane_piece;
   {
     const int Q = lane >> 2, j = lane & 3;  // quad Q of the kilobyte: row 2 * (Q / 4) + Q % 2, one half of its line
     const int row8 = 2 * (Q >> 2) + (Q & 1);
-    const int piece = 4 * (((Q >> 1) & 1) ^ (w & 1)) + ((j - (Q >> 2)) & 3);
+    lane_piece = 4 * (((Q >> 1) & 1) ^ (w & 1)) + ((j - (Q >> 2)) & 3);
 #pragma unroll
     for (int m = 0; m < LA2; m++) {
       const int blk = RS == 1 ? m : min(m, rbt - 1);
-      const int a = rowmap[(rb0 + blk) * kRowBlock + 8 * w + row8];
-      const int tok = a >= 0 ? a / kTopK : 0;  // padding rows read token 0; their products are never used
-      lane_src[m] = (uint32_t)tok * (uint32_t)(KB * 2) + piece;
+      lane_src[m] = (uint32_t)rowmap[(rb0 + blk) * kRowBlock + 8 * w + row8];
     }
   }
   // where this lane finds its operand of (parity of the step, k block) inside a row block's 4 KB
@@ -699,7 +700,7 @@ __device__ __forceinline__ void gemm_tile_gl(const uint4 *__restrict__ x_rows,  
     }
   };
 
-  // A2(0) A2(1) B(0) A2(2) B(1) B(2) A2(3)
+  // one double step of the row operand / one step of the column operand, all of the wave's loads
   auto issue_a2_all = [&](int d, int jd) {
 #pragma unroll
     for (int m = 0; m < LA2; m++) issue_a2(d, min(jd, last_d), m);
@@ -708,21 +709,18 @@ __device__ __forceinline__ void gemm_tile_gl(const uint4 *__restrict__ x_rows,  
 #pragma unroll
     for (int m = 0; m < LB; m++) issue_b(slot, min(ks, last), m);
   };
-  if constexpr (R2 == 4) {  // A2(0) A2(1) B(0) A2(2) B(1) B(2) | A2(3)
-    issue_a2_all(0, 0);
-    issue_a2_all(1, 1);
-    __builtin_amdgcn_sched_barrier(0);  // the counted waits rely on this issue order
-    issue_b_all(0, 0);
-    issue_a2_all(2, 2);
-  } else {  // A2(0) B(0) A2(1) B(1) B(2) | A2(2)
-    issue_a2_all(0, 0);
-    __builtin_amdgcn_sched_barrier(0);
-    issue_b_all(0, 0);
-    issue_a2_all(1, 1);
+  // first filling: B(0) .. B(RB-2), then (the row map has answered meanwhile) A2(0) .. A2(R2-1)
+#pragma unroll
+  for (int k = 0; k < RB - 1; k++) issue_b_all(k, k);
+  __builtin_amdgcn_sched_barrier(0);  // the counted waits rely on this issue order
+#pragma unroll
+  for (int m = 0; m < LA2; m++) {
+    const int a = (int)lane_src[m];
+    const int tok = a >= 0 ? a / kTopK : 0;  // padding rows read token 0; their products are never used
+    lane_src[m] = (uint32_t)tok * (uint32_t)(KB * 2) + lane_piece;
   }
-  __builtin_amdgcn_sched_barrier(0);
-  issue_b_all(1, 1);
-  issue_b_all(2, 2);
+#pragma unroll
+  for (int k = 0; k < R2 - 1; k++) issue_a2_all(k, k);
   __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
   for (int p = 0; p < NBW / 2; p++)
