@@ -445,18 +445,43 @@ __global__ __launch_bounds__(kDispThreads) void dispatch_small_kernel(
 // in place, x = bf16(float(x) + sum) (residual_add_batch_kernel,
 // utility/utility.cpp:158-173; call getp_run.cpp:846-852); inactive rows are
 // left alone.
-template <bool RESID>
+//
+// DIRECT: there was no dispatch pass (see DirectIds).  The row of assignment
+// (t, k) is its expert's slot plus the number of lower assignments of the batch
+// with the same expert, which the workgroup's 256 threads count with a ballot.
+template <bool RESID, bool DIRECT>
 __global__ __launch_bounds__(256) void combine_kernel(const float *__restrict__ y,
                                                      const int *__restrict__ inv,
                                                      const float *__restrict__ topk_v,
                                                      const int *__restrict__ pos, void *outp, int H,
-                                                     int accumulate) {
+                                                     int accumulate, DirectIds ids) {
   const int t = blockIdx.x;
   const bool active = !(pos && pos[t] < 0);
   if (!active && (accumulate || RESID)) return;
   int p[kTopK] = {-1, -1, -1, -1};
   float w[kTopK] = {0.f, 0.f, 0.f, 0.f};
-  if (active) {
+  if (DIRECT) {
+    __shared__ int lower[256 / 64][kTopK];
+    const int tid = threadIdx.x;
+    const int mine = direct_expert_of(ids, tid);
+    int e[kTopK];
+#pragma unroll
+    for (int k = 0; k < kTopK; k++) {
+      e[k] = direct_expert_of(ids, t * kTopK + k);
+      const unsigned long long bal = __ballot(e[k] >= 0 && mine == e[k] && tid < t * kTopK + k);
+      if ((tid & 63) == 0) lower[tid >> 6][k] = __popcll(bal);
+    }
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < kTopK; k++) {
+      const int r = lower[0][k] + lower[1][k] + lower[2][k] + lower[3][k];
+      if (e[k] >= 0 && r < kDirectSlotRows) p[k] = e[k] * kDirectSlotRows + r;
+    }
+    if (active) {
+      const float4 wv = *reinterpret_cast<const float4 *>(topk_v + (size_t)t * kTopK);
+      w[0] = wv.x; w[1] = wv.y; w[2] = wv.z; w[3] = wv.w;
+    }
+  } else if (active) {
     const int4 pi = *reinterpret_cast<const int4 *>(inv + (size_t)t * kTopK);
     const float4 wv = *reinterpret_cast<const float4 *>(topk_v + (size_t)t * kTopK);
     p[0] = pi.x; p[1] = pi.y; p[2] = pi.z; p[3] = pi.w;
@@ -517,14 +542,24 @@ hipError_t launch_dispatch(const int *topk_i, const int *pos, int T, int E, int 
 }
 
 hipError_t launch_combine(const float *y, const int *inv, const float *topk_v, const int *pos,
-                          float *out, int T, int H, int accumulate, hipStream_t s) {
-  combine_kernel<false><<<T, 256, 0, s>>>(y, inv, topk_v, pos, out, H, accumulate);
+                          float *out, int T, int H, int accumulate, const DirectIds &direct,
+                          hipStream_t s) {
+  if (direct.topk_i) {
+    combine_kernel<false, true><<<T, 256, 0, s>>>(y, inv, topk_v, pos, out, H, accumulate, direct);
+  } else {
+    combine_kernel<false, false><<<T, 256, 0, s>>>(y, inv, topk_v, pos, out, H, accumulate, direct);
+  }
   return hipGetLastError();
 }
 
 hipError_t launch_combine_residual(const float *y, const int *inv, const float *topk_v,
-                                   const int *pos, uint16_t *x, int T, int H, hipStream_t s) {
-  combine_kernel<true><<<T, 256, 0, s>>>(y, inv, topk_v, pos, x, H, 0);
+                                   const int *pos, uint16_t *x, int T, int H, const DirectIds &direct,
+                                   hipStream_t s) {
+  if (direct.topk_i) {
+    combine_kernel<true, true><<<T, 256, 0, s>>>(y, inv, topk_v, pos, x, H, 0, direct);
+  } else {
+    combine_kernel<true, false><<<T, 256, 0, s>>>(y, inv, topk_v, pos, x, H, 0, direct);
+  }
   return hipGetLastError();
 }
 

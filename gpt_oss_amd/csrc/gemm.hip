@@ -229,6 +229,7 @@ __device__ __forceinline__ void gemm_tile(const uint4 *__restrict__ a_frag,  // 
                                           const uint16_t *__restrict__ b_scale,  // FP4: expert's [nb/2][KB/2][32] byte pairs
                                           int KB, int rb0, int rbt, int nb0, int nb_valid,
                                           const int *__restrict__ rowmap,    // GATHER: padded row -> assignment
+                                          int map_rb0,                       // row block that rowmap[0] belongs to
                                           const float *__restrict__ bias_a,  // gate / down bias (expert)
                                           const float *__restrict__ bias_b,  // up bias (expert)
                                           void *__restrict__ outp, int out_ld, float limit,
@@ -313,7 +314,7 @@ __device__ __forceinline__ void gemm_tile(const uint4 *__restrict__ a_frag,  // 
     for (int m = 0; m < LA; m++) {
       const int c = min(m * NW + w, A_CH - 1);
       const int blk = RS == 1 ? c / KPS : min(c / KPS, rbt - 1);
-      const int a = rowmap[(rb0 + blk) * kRowBlock + (lane & 31)];
+      const int a = rowmap[(rb0 - map_rb0 + blk) * kRowBlock + (lane & 31)];
       const int tok = a >= 0 ? a / kTopK : 0;
       lane_off[m] = (uint32_t)tok * (uint32_t)(KB * 2) + (c % KPS) * 2 + (lane >> 5);
     }
@@ -810,14 +811,21 @@ __device__ __forceinline__ void gemm_tile_gl(const uint4 *__restrict__ x_rows,  
   gate_up_epilogue<RBT, RS, C>(acc, outp, out_ld, limit, rb0, rbt, nb0, nb_valid, cw, rg, lane);
 }
 
-template <typename C, bool GATE_UP, bool FP4, bool GATHER>
+// DIRECT (small-batch configuration only): there is no plan.  Workgroup b is
+// column tile b % n_ct of expert b / n_ct; its 256 threads look at one
+// assignment of the batch each and find the expert's rows with a ballot (see
+// DirectIds).  An expert without rows ends its workgroups here.
+template <typename C, bool GATE_UP, bool FP4, bool GATHER, bool DIRECT = false>
 __global__ __launch_bounds__(C::THREADS, C::WAVES) void grouped_gemm_kernel(
     const uint4 *__restrict__ a_frag, const uint4 *__restrict__ w_frag,
     const uint16_t *__restrict__ w_scale,
     const float *__restrict__ bias_a, const float *__restrict__ bias_b,
     const TileDesc *__restrict__ tiles, const int *__restrict__ totals,
-    const int *__restrict__ rowmap, void *__restrict__ outp, int K, int N, float limit) {
+    const int *__restrict__ rowmap, void *__restrict__ outp, int K, int N, float limit,
+    DirectIds ids) {
   static_assert(!GATHER || GATE_UP, "only the first GEMM reads token rows");
+  static_assert(!DIRECT || (C::RBT_MAX * kRowBlock == kDirectSlotRows && C::THREADS == kDirectTokens * kTopK),
+                "a direct batch: one thread per assignment, an expert's slot is one tile high");
   constexpr int R = C::R;
   static_assert(R <= 7, "seven stage arrays are declared below");
   __shared__ uint4 st0[C::STAGE], st1[C::STAGE], st2[C::STAGE], st3[C::STAGE], st4[C::STAGE],
@@ -827,7 +835,39 @@ __global__ __launch_bounds__(C::THREADS, C::WAVES) void grouped_gemm_kernel(
   const int nb_total = (GATE_UP ? 2 * N : N) / kRowBlock;  // weight row blocks per expert
   const int n_ct = (nb_total + C::TILE_NB - 1) / C::TILE_NB;
   TileDesc tc;
-  if (!locate_tile(tiles, totals + (GATE_UP ? kTotBoundsGateUp : kTotBoundsDown), tc)) return;
+  __shared__ int direct_rows[kDirectSlotRows];  // slot row -> assignment, -1 = padding
+  __shared__ int direct_cnt[C::NW];
+  const int *map = rowmap;
+  if constexpr (DIRECT) {
+    const int tid = threadIdx.x;
+    const int e = blockIdx.x / n_ct;
+    const bool mine = direct_expert_of(ids, tid) == e;
+    const unsigned long long bal = __ballot(mine);
+    if ((tid & 63) == 0) direct_cnt[tid >> 6] = __popcll(bal);
+    if (tid < kDirectSlotRows) direct_rows[tid] = -1;
+    __syncthreads();
+    int before = 0, count = 0;
+#pragma unroll
+    for (int ww = 0; ww < C::NW; ww++) {
+      const int c = direct_cnt[ww];
+      if (ww < (tid >> 6)) before += c;
+      count += c;
+    }
+    if (count == 0) return;
+    if (GATHER) {
+      const int r = before + __popcll(bal & ((1ull << (tid & 63)) - 1ull));
+      if (mine && r < kDirectSlotRows) direct_rows[r] = tid;
+      __syncthreads();
+      map = direct_rows;
+    }
+    tc.e = e;
+    tc.nt = blockIdx.x % n_ct;
+    tc.rb0 = e * (kDirectSlotRows / kRowBlock);
+    tc.rbt = (min(count, kDirectSlotRows) + kRowBlock - 1) / kRowBlock;
+  } else {
+    if (!locate_tile(tiles, totals + (GATE_UP ? kTotBoundsGateUp : kTotBoundsDown), tc)) return;
+  }
+  const int map_rb0 = DIRECT ? tc.rb0 : 0;
   const int nb0 = tc.nt * C::TILE_NB;
   const int nb_valid = min(C::TILE_NB, nb_total - nb0);
   // per expert: bf16 nb_total * KB fragments of 1 KB; MXFP4 (nb_total/2) * (KB/2) chunks of 1 KB
@@ -844,8 +884,8 @@ __global__ __launch_bounds__(C::THREADS, C::WAVES) void grouped_gemm_kernel(
                                   outp, N, limit, st0, st1, st2, st3, st4, st5, st6, st7);                    \
     } else {                                                                                                  \
       gemm_tile<n, rs, C, GATE_UP, FP4, GATHER>(a_frag, b_frag, b_scale, KB, tc.rb0, tc.rbt, nb0, nb_valid,   \
-                                                rowmap, ba, bb, outp, N, limit, st0, st1, st2, st3, st4, st5, \
-                                                st6, epi);                                                    \
+                                                map, map_rb0, ba, bb, outp, N, limit, st0, st1, st2, st3,     \
+                                                st4, st5, st6, epi);                                          \
     }                                                                                                         \
   } while (0)
 #define MOE_TILE(n) MOE_TILE_RS(n, 1)
@@ -898,47 +938,52 @@ constexpr int kSmallBatchTokens = CfgGemmSmall::RBT_MAX * kRowBlock;
 
 // w_scale == nullptr: w holds bf16 fragments; otherwise w holds MXFP4 chunks and
 // w_scale their scale bytes (pack_fp4_kernel).
-template <typename C, bool GATE_UP, bool GATHER = false>
+template <typename C, bool GATE_UP, bool GATHER = false, bool DIRECT = false>
 static hipError_t launch_gemm(const uint4 *a, const uint4 *w, const uint16_t *w_scale, const float *ba,
                               const float *bb, const DispatchBuffers &d, void *out, int K, int N,
-                              float limit, int mt_cap, hipStream_t s) {
+                              float limit, int mt_cap, const DirectIds &direct, hipStream_t s) {
   const int nb_total = (GATE_UP ? 2 * N : N) / kRowBlock;
   const int n_ct = (nb_total + C::TILE_NB - 1) / C::TILE_NB;
-  const int grid = kXcds * xcd_tile_cap(mt_cap * n_ct);
+  const int grid = DIRECT ? direct.E * n_ct : kXcds * xcd_tile_cap(mt_cap * n_ct);
   const TileDesc *tiles = GATE_UP ? d.tiles_gate_up : d.tiles_down;
   if (w_scale) {
-    grouped_gemm_kernel<C, GATE_UP, true, GATHER><<<grid, C::THREADS, 0, s>>>(
-        a, w, w_scale, ba, bb, tiles, d.totals, d.rowmap, out, K, N, limit);
+    grouped_gemm_kernel<C, GATE_UP, true, GATHER, DIRECT><<<grid, C::THREADS, 0, s>>>(
+        a, w, w_scale, ba, bb, tiles, d.totals, d.rowmap, out, K, N, limit, direct);
   } else {
-    grouped_gemm_kernel<C, GATE_UP, false, GATHER><<<grid, C::THREADS, 0, s>>>(
-        a, w, nullptr, ba, bb, tiles, d.totals, d.rowmap, out, K, N, limit);
+    grouped_gemm_kernel<C, GATE_UP, false, GATHER, DIRECT><<<grid, C::THREADS, 0, s>>>(
+        a, w, nullptr, ba, bb, tiles, d.totals, d.rowmap, out, K, N, limit, direct);
   }
   return hipGetLastError();
 }
 
 hipError_t launch_gate_up(const uint16_t *x, const void *w1, const uint16_t *w1_scale, const float *b1g,
                           const float *b1u, const DispatchBuffers &d, uint16_t *act, int H, int IM,
-                          float limit, int mt_cap, int max_rows, hipStream_t s) {
+                          float limit, int mt_cap, int max_rows, const DirectIds &direct, hipStream_t s) {
   static_assert(kSmallBatchTokens == kSmallBatchRows, "small_batch() and the small-batch configuration");
   const uint4 *w = reinterpret_cast<const uint4 *>(w1);
   const uint4 *rows = reinterpret_cast<const uint4 *>(x);
+  if (direct.topk_i)
+    return launch_gemm<CfgGemmSmall, true, true, true>(rows, w, w1_scale, b1g, b1u, d, act, H, IM, limit,
+                                                       mt_cap, direct, s);
   // either way the row operand is read from the token rows: 32 bytes of 32 rows per
   // instruction in the small-batch configuration, whole lines of 8 rows otherwise
   if (small_batch(max_rows))
-    return launch_gemm<CfgGemmSmall, true, true>(rows, w, w1_scale, b1g, b1u, d, act, H, IM, limit, mt_cap, s);
-  return launch_gemm<CfgGemm, true, true>(rows, w, w1_scale, b1g, b1u, d, act, H, IM, limit, mt_cap, s);
+    return launch_gemm<CfgGemmSmall, true, true>(rows, w, w1_scale, b1g, b1u, d, act, H, IM, limit, mt_cap,
+                                                 direct, s);
+  return launch_gemm<CfgGemm, true, true>(rows, w, w1_scale, b1g, b1u, d, act, H, IM, limit, mt_cap, direct, s);
 }
 
 hipError_t launch_down(const uint16_t *act, const void *w2, const uint16_t *w2_scale, const float *b2,
                        const DispatchBuffers &d, float *y, int H, int IM, int mt_cap, int max_rows,
-                       hipStream_t s) {
-  if (max_rows <= kSmallBatchTokens)
-    return launch_gemm<CfgGemmSmall, false>(reinterpret_cast<const uint4 *>(act),
-                                            reinterpret_cast<const uint4 *>(w2), w2_scale, b2, nullptr,
-                                            d, y, IM, H, 0.f, mt_cap, s);
-  return launch_gemm<CfgGemm, false>(reinterpret_cast<const uint4 *>(act),
-                                     reinterpret_cast<const uint4 *>(w2), w2_scale, b2, nullptr, d, y,
-                                     IM, H, 0.f, mt_cap, s);
+                       const DirectIds &direct, hipStream_t s) {
+  const uint4 *a = reinterpret_cast<const uint4 *>(act);
+  const uint4 *w = reinterpret_cast<const uint4 *>(w2);
+  if (direct.topk_i)
+    return launch_gemm<CfgGemmSmall, false, false, true>(a, w, w2_scale, b2, nullptr, d, y, IM, H, 0.f,
+                                                         mt_cap, direct, s);
+  if (small_batch(max_rows))
+    return launch_gemm<CfgGemmSmall, false>(a, w, w2_scale, b2, nullptr, d, y, IM, H, 0.f, mt_cap, direct, s);
+  return launch_gemm<CfgGemm, false>(a, w, w2_scale, b2, nullptr, d, y, IM, H, 0.f, mt_cap, direct, s);
 }
 
 }  // namespace moe

@@ -65,6 +65,9 @@ struct moe_handle {
   int a_pad_cap = 0;  // max padded rows
   int n_blk_cap = 0;
   int disp_tokens = -1;  // batch of the last moe_dispatch (stage-level calls), -1: none
+  // The last call ran without a dispatch pass (at most 64 tokens): its ids, for a
+  // moe_get_dispatch that asks for the plan afterwards.  topk_i == nullptr: none.
+  DirectIds unplanned{nullptr, nullptr, 0, 0};
   // expert pipeline
   uint16_t *act = nullptr;  // SwiGLU output, bf16 fragments
   float *y = nullptr;       // down output [a_pad_cap, H]
@@ -137,30 +140,30 @@ inline int down_col_tiles(const moe_config &c) {
 // reads the routed token rows itself, there is no gathered copy), down GEMM.
 // Leaves the per-assignment rows in h->y.
 // max_rows: no expert is given more rows than this (T when the ids of a token are distinct).
-int run_gemms(moe_handle *h, int layer, const uint16_t *x, int T, int max_rows, hipStream_t s,
-              StageTimer &tm) {
+int run_gemms(moe_handle *h, int layer, const uint16_t *x, int T, int max_rows, const DirectIds &direct,
+              hipStream_t s, StageTimer &tm) {
   const moe_config &c = h->cfg;
   const LayerWeights &lw = h->layers[layer];
   const int A = T * kTopK;
   const int mt_cap = A / kTileRows + c.experts;
   HIP_TRY(tm.mark(MOE_STAGE_GATE_UP));
   HIP_TRY(launch_gate_up(x, lw.w1q ? static_cast<const void *>(lw.w1q) : lw.w1, lw.w1s, lw.b1g, lw.b1u,
-                         h->disp, h->act, c.hidden, c.inter, c.swiglu_limit, mt_cap, max_rows, s));
+                         h->disp, h->act, c.hidden, c.inter, c.swiglu_limit, mt_cap, max_rows, direct, s));
   HIP_TRY(tm.mark(MOE_STAGE_DOWN));
   HIP_TRY(launch_down(h->act, lw.w2q ? static_cast<const void *>(lw.w2q) : lw.w2, lw.w2s, lw.b2,
-                      h->disp, h->y, c.hidden, c.inter, mt_cap, max_rows, s));
+                      h->disp, h->y, c.hidden, c.inter, mt_cap, max_rows, direct, s));
   return MOE_OK;
 }
 
 // Stage 6: out != nullptr: out (+)= sum_k w[t,k] * y[row of (t,k)], fp32.
 // Otherwise resid (bf16, in place) += that sum.
 int run_combine(moe_handle *h, const float *topk_v, const int *pos, int T, float *out, int accumulate,
-                uint16_t *resid, hipStream_t s, StageTimer &tm) {
+                uint16_t *resid, const DirectIds &direct, hipStream_t s, StageTimer &tm) {
   HIP_TRY(tm.mark(MOE_STAGE_COMBINE));
   if (out) {
-    HIP_TRY(launch_combine(h->y, h->disp.inv, topk_v, pos, out, T, h->cfg.hidden, accumulate, s));
+    HIP_TRY(launch_combine(h->y, h->disp.inv, topk_v, pos, out, T, h->cfg.hidden, accumulate, direct, s));
   } else {
-    HIP_TRY(launch_combine_residual(h->y, h->disp.inv, topk_v, pos, resid, T, h->cfg.hidden, s));
+    HIP_TRY(launch_combine_residual(h->y, h->disp.inv, topk_v, pos, resid, T, h->cfg.hidden, direct, s));
   }
   HIP_TRY(tm.mark(MOE_NUM_STAGES));
   return MOE_OK;
@@ -172,11 +175,17 @@ int run_experts(moe_handle *h, int layer, const uint16_t *x, const int *pos, con
                 StageTimer &tm, uint16_t *resid = nullptr) {
   const moe_config &c = h->cfg;
   HIP_TRY(tm.mark(MOE_STAGE_DISPATCH));
-  HIP_TRY(launch_dispatch(topk_i, pos, T, c.experts, gate_up_col_tiles(c), down_col_tiles(c), h->disp, s));
+  // a batch of at most 64 tokens needs no dispatch pass: the GEMMs and the
+  // combine find their rows from the ids themselves
+  const bool direct_plan = direct_plan_fits(T, max_rows, c.experts, h->a_pad_cap);
+  const DirectIds direct{direct_plan ? topk_i : nullptr, pos, T, c.experts};
+  if (!direct_plan)
+    HIP_TRY(launch_dispatch(topk_i, pos, T, c.experts, gate_up_col_tiles(c), down_col_tiles(c), h->disp, s));
+  h->unplanned = direct;
   h->disp_tokens = -1;  // the plan now belongs to this call, not to a moe_dispatch
-  int rc = run_gemms(h, layer, x, T, max_rows, s, tm);
+  int rc = run_gemms(h, layer, x, T, max_rows, direct, s, tm);
   if (rc != MOE_OK) return rc;
-  return run_combine(h, topk_v, pos, T, out, accumulate, resid, s, tm);
+  return run_combine(h, topk_v, pos, T, out, accumulate, resid, direct, s, tm);
 }
 
 }  // namespace
@@ -217,6 +226,8 @@ int moe_create(const moe_config *cfg, moe_handle **out) {
   const int E = cfg->experts, H = cfg->hidden, IM = cfg->inter, T = cfg->max_tokens;
   h->a_cap = T * kTopK;
   h->a_pad_cap = ((h->a_cap + kTileGran * E + kTileGran - 1) / kTileGran) * kTileGran;
+  // room for the fixed slots of the batches that run without a dispatch pass
+  if (h->a_pad_cap < kDirectSlotRows * E) h->a_pad_cap = kDirectSlotRows * E;
   h->n_blk_cap = (T + 255) / 256;
   int rc = MOE_OK;
 #define ALLOC(ptr, count)                                   \
@@ -438,6 +449,7 @@ int moe_dispatch(moe_handle *h, const int *topk_i, const int *pos, int n_tokens,
   HIP_TRY(launch_dispatch(topk_i, pos, n_tokens, h->cfg.experts, gate_up_col_tiles(h->cfg),
                           down_col_tiles(h->cfg), h->disp, static_cast<hipStream_t>(stream)));
   h->disp_tokens = n_tokens;
+  h->unplanned.topk_i = nullptr;
   return MOE_OK;
 }
 
@@ -446,6 +458,12 @@ int moe_get_dispatch(moe_handle *h, int *offsets, int *perm, int n_tokens, void 
   if (n_tokens < 0 || n_tokens > h->cfg.max_tokens)
     return fail(MOE_ERR_BAD_ARG, "n_tokens %d out of range", n_tokens);
   hipStream_t s = static_cast<hipStream_t>(stream);
+  if (h->unplanned.topk_i) {
+    const moe_config &c = h->cfg;
+    HIP_TRY(launch_dispatch(h->unplanned.topk_i, h->unplanned.pos, h->unplanned.T, c.experts,
+                            gate_up_col_tiles(c), down_col_tiles(c), h->disp, s));
+    h->unplanned.topk_i = nullptr;
+  }
   if (offsets)
     HIP_TRY(hipMemcpyAsync(offsets, h->disp.offsets, ((size_t)h->cfg.experts + 1) * sizeof(int),
                            hipMemcpyDeviceToDevice, s));
@@ -481,7 +499,7 @@ int moe_expert_gemms(moe_handle *h, int layer, const uint16_t *x, int n_tokens, 
   StageTimer tm(h, nullptr);  // stage-level calls are not timed
   tm.ev = nullptr;
   // the ids of a moe_dispatch come from outside and may name an expert in several slots of a token
-  return run_gemms(h, layer, x, n_tokens, n_tokens * kTopK, s, tm);
+  return run_gemms(h, layer, x, n_tokens, n_tokens * kTopK, DirectIds{nullptr, nullptr, 0, 0}, s, tm);
 }
 
 int moe_combine(moe_handle *h, const float *topk_v, const int *pos, int n_tokens, float *out,
@@ -495,7 +513,8 @@ int moe_combine(moe_handle *h, const float *topk_v, const int *pos, int n_tokens
   if (!topk_v || !out) return fail(MOE_ERR_BAD_ARG, "null device pointer");
   StageTimer tm(h, nullptr);
   tm.ev = nullptr;
-  return run_combine(h, topk_v, pos, n_tokens, out, accumulate, nullptr, static_cast<hipStream_t>(stream), tm);
+  return run_combine(h, topk_v, pos, n_tokens, out, accumulate, nullptr, DirectIds{nullptr, nullptr, 0, 0},
+                     static_cast<hipStream_t>(stream), tm);
 }
 
 int moe_forward(moe_handle *h, int layer, const uint16_t *x, const int *pos, int n_tokens,

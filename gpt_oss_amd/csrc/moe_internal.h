@@ -131,6 +131,33 @@ struct DispatchBuffers {
 };
 hipError_t launch_dispatch(const int *topk_i, const int *pos, int T, int E, int n_ct_gate_up,
                            int n_ct_down, const DispatchBuffers &d, hipStream_t s);
+
+// Batches of at most kDirectTokens tokens run without a dispatch pass: the 256
+// threads of a workgroup hold one assignment each, so every workgroup of the
+// GEMMs and of the combine reads the batch's expert ids itself and finds its
+// rows with a ballot.  Expert e owns the padded rows [e * kDirectSlotRows,
+// (e + 1) * kDirectSlotRows); inside them its assignments stand in ascending
+// order, as the dispatch kernels place them.  Requires that no expert is given
+// more than kDirectSlotRows assignments.  topk_i == nullptr: not in use, the
+// plan of launch_dispatch is.
+constexpr int kDirectTokens = 64;
+constexpr int kDirectSlotRows = 64;
+struct DirectIds {
+  const int *topk_i;  // [T, 4]
+  const int *pos;     // [T] or nullptr
+  int T, E;
+};
+// expert of assignment a by the rule of the dispatch kernels: -1 past the batch,
+// for a row with pos < 0 and for an id outside [0, E)
+__device__ __forceinline__ int direct_expert_of(const DirectIds &d, int a) {
+  if (a >= d.T * kTopK) return -1;
+  const int id = d.topk_i[a];                      // both loads go out together
+  const int ps = d.pos ? d.pos[a / kTopK] : 0;
+  return ps >= 0 && id >= 0 && id < d.E ? id : -1;
+}
+inline bool direct_plan_fits(int T, int max_rows, int E, int a_pad_cap) {
+  return T <= kDirectTokens && max_rows <= kDirectSlotRows && kDirectSlotRows * E <= a_pad_cap;
+}
 // gate_up reads the routed token rows of x itself, through rowmap; there is no
 // gathered copy.  Batches in which no expert has more than kSmallBatchRows rows
 // run the small-batch configuration of both GEMMs.
@@ -138,14 +165,17 @@ constexpr int kSmallBatchRows = 64;
 inline bool small_batch(int max_rows) { return max_rows <= kSmallBatchRows; }
 hipError_t launch_gate_up(const uint16_t *x, const void *w1, const uint16_t *w1_scale, const float *b1g,
                           const float *b1u, const DispatchBuffers &d, uint16_t *act, int H, int IM,
-                          float limit, int mt_cap, int max_rows, hipStream_t s);
+                          float limit, int mt_cap, int max_rows, const DirectIds &direct, hipStream_t s);
 hipError_t launch_down(const uint16_t *act, const void *w2, const uint16_t *w2_scale, const float *b2,
                        const DispatchBuffers &d, float *y, int H, int IM, int mt_cap, int max_rows,
-                       hipStream_t s);
+                       const DirectIds &direct, hipStream_t s);
+// direct.topk_i != nullptr: the rows of y are found from the ids (inv is not read)
 hipError_t launch_combine(const float *y, const int *inv, const float *topk_v, const int *pos,
-                          float *out, int T, int H, int accumulate, hipStream_t s);
+                          float *out, int T, int H, int accumulate, const DirectIds &direct,
+                          hipStream_t s);
 hipError_t launch_combine_residual(const float *y, const int *inv, const float *topk_v,
-                                   const int *pos, uint16_t *x, int T, int H, hipStream_t s);
+                                   const int *pos, uint16_t *x, int T, int H, const DirectIds &direct,
+                                   hipStream_t s);
 hipError_t launch_rmsnorm(const uint16_t *x, const float *weight, const int *pos, uint16_t *t_out,
                           int T, int H, hipStream_t s);
 

@@ -155,7 +155,11 @@ int moe_dispatch(moe_handle *h, const int *topk_i, const int *pos, int n_tokens,
 
 /* Copies the result of the last dispatch to device buffers of the caller:
  * offsets int [E+1], perm int [n_tokens*K] (entries past offsets[E] are -1).
- * Either may be NULL. */
+ * Either may be NULL.  The last dispatch is that of moe_dispatch or of the last
+ * moe_forward / moe_experts / moe_block_forward.  Those three need no dispatch
+ * pass for a batch of at most 64 tokens; after such a call this function runs
+ * it, on `stream`, from the ids and pos of that call, which must still be
+ * valid (moe_forward and moe_block_forward keep their ids in the handle). */
 int moe_get_dispatch(moe_handle *h, int *offsets, int *perm, int n_tokens,
                      void *stream);
 

@@ -385,6 +385,48 @@ def test_c5_mxfp4_ingest():
         m4.upload_layer_mxfp4(3, wr, br, b1k, s1, b1, b2k, s2, b2)  # layer out of range
 
 
+@pytest.mark.parametrize("T", [5, 33, 64])
+def test_small_batches_without_dispatch_pass(c2, T):
+    """Up to 64 tokens moe_forward launches no dispatch kernels: the workgroups
+    of the GEMMs and of the combine find their rows from the expert ids
+    themselves, in fixed slots of 64 rows per expert.  The staged entry points
+    (moe_dispatch, moe_expert_gemms, moe_combine) keep the planned path, so the
+    same batch through both must give the same bits -- with inactive rows too,
+    which come out as zeros, are left alone in accumulate mode, and whose
+    removal from the batch changes nothing for the others."""
+    sh, L, m = c2
+    H = sh.hidden
+    x = L["x"][900:900 + T]
+    pos = np.where(np.random.default_rng(T).random(T) < 0.3, -1, 3).astype(np.int32)
+    pos[0] = 3
+    for p in (None, pos):
+        R = abi.run_layer(m, 0, x, p)
+        check_routing(R, L, x, p, sh.experts)
+        rows = np.arange(T) if p is None else np.nonzero(p >= 0)[0]
+        check_outputs(R, L, x, p, rows[:24])
+        dx = abi.DevBuf.from_numpy(synth.to_bf16_bits(x))
+        dpos = abi.DevBuf.from_numpy(p) if p is not None else None
+        dti, dtv = abi.DevBuf.from_numpy(R["topk_i"]), abi.DevBuf.from_numpy(R["topk_v"])
+        m.dispatch(dti, dpos, T)
+        m.expert_gemms(0, dx, T)
+        dout = abi.DevBuf(T * H * 4)
+        dout.memset(0xFF)
+        m.combine(dtv, dpos, T, dout, accumulate=False)
+        abi.sync()
+        assert np.array_equal(dout.download((T, H), np.float32), R["out"])
+    a = R["out"]
+    assert np.all(a[pos < 0] == 0)
+    b = abi.run_layer(m, 0, np.ascontiguousarray(x[pos >= 0]), None)["out"]
+    assert np.array_equal(a[pos >= 0], b)
+    prior = np.random.default_rng(4).standard_normal((T, H)).astype(np.float32)
+    dout = abi.DevBuf.from_numpy(prior)
+    m.forward(0, dx, dpos, T, dout, accumulate=True)
+    abi.sync()
+    got = dout.download((T, H), np.float32)
+    assert np.array_equal(got[pos < 0], prior[pos < 0])
+    np.testing.assert_allclose(got[pos >= 0], prior[pos >= 0] + a[pos >= 0], rtol=0, atol=1e-6)
+
+
 def test_small_batches_repeat_bit_for_bit():
     """Batches of at most 64 tokens take paths of their own (one-workgroup
     dispatch, gate_up reading the token rows through the row map, GEMMs built
