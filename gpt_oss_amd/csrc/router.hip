@@ -92,6 +92,67 @@ __device__ __forceinline__ float4 softmax4(const float (&v)[kTopK]) {
                      (float)((double)ev[2] / sum), (float)((double)ev[3] / sum));
 }
 
+// Top-NSEL of one token's logits for up to 32 experts, one lane per expert (the
+// 32 lanes of a half wave; lane e owns expert e, v = its logit, -inf for a lane
+// without an expert).  row4 points at the token's E_pad logits in LDS, 16-byte
+// aligned.  Same rule as select_top, found by counting instead of five rounds
+// of comparisons: an expert's place is the number of experts with a greater
+// value; the lanes at places 0 .. NSEL-1 post themselves to `post` (LDS, NSEL
+// floats then NSEL ints, owned by this token) and every lane reads the list
+// back.  Of experts with equal values the lowest index takes the place (an
+// atomic minimum) and the place behind it stays empty: an empty place among the
+// first NSEL, like a NaN among the logits (which no count orders), sends the
+// wave -- the branch is per wave -- through select_top's comparison-by-
+// comparison rule instead.  Places past the number of experts hold kNone.
+template <int E_pad, int NSEL>
+__device__ __forceinline__ void ranked_top(const float4 *row4, float v, int e, int E, float *post,
+                                           float (&sel_v)[NSEL], int (&sel_i)[NSEL]) {
+  static_assert(E_pad == 16 || E_pad == 32, "one lane per expert in a half wave");
+  int *post_i = reinterpret_cast<int *>(post + NSEL);
+  if (e < NSEL) post_i[e] = kNone;
+  int place = 0;
+#pragma unroll
+  for (int j4 = 0; j4 < E_pad / 4; j4++) {
+    const float4 o = row4[j4];  // the same address in all lanes of the half wave
+    place += (o.x > v ? 1 : 0) + (o.y > v ? 1 : 0) + (o.z > v ? 1 : 0) + (o.w > v ? 1 : 0);
+  }
+  if (e < E && place < NSEL) {
+    post[place] = v;  // equal values: the same float from every writer
+    atomicMin(&post_i[place], e);
+  }
+  // the same wave wrote the list; LDS operations of a wave complete in order
+  bool redo = v != v;
+#pragma unroll
+  for (int r = 0; r < NSEL; r++) {
+    sel_v[r] = post[r];
+    sel_i[r] = post_i[r];
+    redo |= r < E && sel_i[r] == kNone;
+  }
+  if (__ballot(redo) != 0ull) {
+    const float own[1] = {v};
+    select_top<1, 32, NSEL>(own, e, E, sel_v, sel_i);
+  }
+}
+
+// The softmax of run.cpp:336-354 over the four selected logits with the work
+// spread over four lanes of the token (lane r < 4 computes exp and quotient of
+// place r; the sum is formed in every lane in the order of the reference), and
+// the token's ids and weights stored by those lanes.  base = the token's first
+// lane in the wave.
+__device__ __forceinline__ void store_topk_spread(const float (&v)[kTopK], const int (&id)[kTopK], int r,
+                                                  int base, int *topk_i_row, float *topk_v_row) {
+  const double mx = (double)v[0];
+  const float mine = r == 0 ? v[0] : (r == 1 ? v[1] : (r == 2 ? v[2] : v[3]));
+  const float ev = expf((float)((double)mine - mx));
+  double sum = 0.0;
+#pragma unroll
+  for (int k = 0; k < kTopK; k++) sum += (double)__shfl(ev, base + k, 64);
+  if (r < kTopK) {
+    topk_i_row[r] = r == 0 ? id[0] : (r == 1 ? id[1] : (r == 2 ? id[2] : id[3]));
+    topk_v_row[r] = (float)((double)ev / sum);
+  }
+}
+
 __device__ __forceinline__ void unpack8(const uint4 v, float (&f)[8]) {
   f[0] = __uint_as_float(v.x << 16); f[1] = __uint_as_float(v.x & 0xffff0000u);
   f[2] = __uint_as_float(v.y << 16); f[3] = __uint_as_float(v.y & 0xffff0000u);
@@ -110,18 +171,22 @@ __global__ __launch_bounds__(WPC * 64) void router_kernel(
     float *__restrict__ score, int *__restrict__ topk_i, float *__restrict__ topk_v) {
   constexpr int E_pad = NT * 16;
   constexpr int TOK = MT * 16;
-  // selection: LPT lanes per token, each owning PER experts; SW waves take part
-  constexpr int LPT = E_pad <= 64 ? 4 : (E_pad == 128 ? 8 : 16);
-  constexpr int PER = E_pad / LPT;
+  // selection: LPT lanes per token, each owning PER experts; SW waves take part.
+  // Up to 32 experts: one lane per expert, places found by counting (ranked_top).
+  constexpr bool RANKED = E_pad <= 32;
+  constexpr int LPT = RANKED ? 32 : (E_pad <= 64 ? 4 : (E_pad == 128 ? 8 : 16));
+  constexpr int PER = RANKED ? 1 : E_pad / LPT;
   constexpr int SW = TOK * LPT / 64;
   static_assert(SW >= 1 && SW <= WPC, "waves of the selection");
+  constexpr int LOG_LD = RANKED ? E_pad + 4 : E_pad + 1;  // RANKED reads rows of logits in 16-byte pieces
   // cross-wave sum: GB blocks of 16 x 16 outputs at a time through 32 KB
   constexpr int NBLK = MT * NT;
   constexpr int GB = 32 / WPC < NBLK ? 32 / WPC : NBLK;
   static_assert(WPC >= 2 && NBLK % GB == 0, "groups of the cross-wave sum");
   __shared__ double part[WPC / 2][GB][4][64];  // [wave][block][reg][lane]
   __shared__ float sumsq[WPC][TOK];
-  __shared__ float logits[TOK][E_pad + 1];
+  __shared__ __attribute__((aligned(16))) float logits[TOK][LOG_LD];
+  __shared__ float posted[RANKED ? TOK : 1][2 * (kTopK + 1)];  // ranked_top's lists
   __shared__ unsigned short tasks[TOK * E_pad];  // (token in tile) * E_pad + expert
   __shared__ int n_tasks;
   __shared__ float sh_br[E_pad];  // the bias, fetched while the first pass runs
@@ -255,11 +320,17 @@ __global__ __launch_bounds__(WPC * 64) void router_kernel(
   bool undecided = false;
   if (w < SW) {
     float v[PER];
-#pragma unroll
-    for (int j = 0; j < PER; j++) v[j] = logits[tr][q * PER + j];
     float s_v[kTopK + 1];
     int s_i[kTopK + 1];
-    select_top<PER, LPT, kTopK + 1>(v, q, E, s_v, s_i);
+    if constexpr (RANKED) {
+      v[0] = q < E_pad ? logits[tr][q] : -__builtin_inff();
+      ranked_top<E_pad, kTopK + 1>(reinterpret_cast<const float4 *>(&logits[tr][0]), v[0], q, E, posted[tr],
+                                   s_v, s_i);
+    } else {
+#pragma unroll
+      for (int j = 0; j < PER; j++) v[j] = logits[tr][q * PER + j];
+      select_top<PER, LPT, kTopK + 1>(v, q, E, s_v, s_i);
+    }
     if (active) {
       float ss = 0.f;
 #pragma unroll
@@ -272,7 +343,13 @@ __global__ __launch_bounds__(WPC * 64) void router_kernel(
       const bool decided = lo(s_v[0]) > up(s_v[1]) && lo(s_v[1]) > up(s_v[2]) && lo(s_v[2]) > up(s_v[3]) &&
                            (s_i[4] == kNone || lo(s_v[3]) > up(s_v[4]));
       if (decided) {
-        if (q == 0) {
+        if constexpr (RANKED) {
+          // (tokens of one wave can differ in `decided`: the shuffles inside are
+          // among the lanes of one token, which agree)
+          const float sv[kTopK] = {s_v[0], s_v[1], s_v[2], s_v[3]};
+          const int si[kTopK] = {s_i[0], s_i[1], s_i[2], s_i[3]};
+          store_topk_spread(sv, si, q, lane - q, topk_i + (size_t)t * kTopK, topk_v + (size_t)t * kTopK);
+        } else if (q == 0) {
           const float sv[kTopK] = {s_v[0], s_v[1], s_v[2], s_v[3]};
           *reinterpret_cast<int4 *>(topk_i + (size_t)t * kTopK) = make_int4(s_i[0], s_i[1], s_i[2], s_i[3]);
           *reinterpret_cast<float4 *>(topk_v + (size_t)t * kTopK) = softmax4(sv);
@@ -354,7 +431,15 @@ __global__ __launch_bounds__(WPC * 64) void router_kernel(
   }
   __syncthreads();
 
-  if (undecided) {  // waves < SW only
+  if constexpr (RANKED) {
+    if (w < SW && __ballot(undecided) != 0ull) {  // per wave: ranked_top is a wave's work
+      const float v = q < E_pad ? logits[tr][q] : -__builtin_inff();
+      float s_v[kTopK];
+      int s_i[kTopK];
+      ranked_top<E_pad, kTopK>(reinterpret_cast<const float4 *>(&logits[tr][0]), v, q, E, posted[tr], s_v, s_i);
+      if (undecided) store_topk_spread(s_v, s_i, q, lane - q, topk_i + (size_t)t * kTopK, topk_v + (size_t)t * kTopK);
+    }
+  } else if (undecided) {  // waves < SW only
     float v[PER];
 #pragma unroll
     for (int j = 0; j < PER; j++) v[j] = logits[tr][q * PER + j];
