@@ -41,7 +41,8 @@
 // with the row tile fastest, and XCD x takes a contiguous range of them (see
 // dispatch_scan_kernel: about an eighth by estimated cost): the tiles an XCD
 // runs at one time share the expert's rows and a few column slabs of its
-// weights, so each weight byte leaves HBM once.
+// weights, so each weight byte leaves HBM once.  (Batches of at most 64 tokens
+// have no tile table at all: see DIRECT at the kernel.)
 #include <type_traits>
 #include <utility>
 
