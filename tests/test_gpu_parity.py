@@ -183,6 +183,14 @@ def test_dispatch_bit_exact(E):
     _dispatch_case(m, ti, None, E)
     # nothing active
     _dispatch_case(m, ti, np.full(T, -1, np.int32), E)
+    # a batch beyond the benchmark sizes: 36 workgroups in the count and scatter passes
+    m.close()
+    T = 9000
+    m = abi.Moe(64, 64, E, max_tokens=T)
+    ti = np.stack([rng.permutation(E)[:4] for _ in range(T)]).astype(np.int32)
+    pos = np.where(rng.random(T) < 0.15, -1, 1).astype(np.int32)
+    _dispatch_case(m, ti, pos, E)
+    m.close()
 
 
 # ---------------- whole layer at the benchmark shapes ----------------
