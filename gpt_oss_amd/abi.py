@@ -23,10 +23,11 @@ SYMBOLS = [
     "moe_forward", "moe_block_forward",
     "moe_router",
     "moe_dispatch", "moe_get_dispatch", "moe_experts", "moe_expert_gemms", "moe_combine",
-    "moe_dispatch_static", "moe_profile_enable",
+    "moe_dispatch_static", "moe_set_distinct_ids", "moe_profile_enable",
     "moe_profile_read", "moe_weight_bytes", "moe_workspace_bytes", "moe_last_error",
     "moe_version", "moe_dev_alloc", "moe_dev_free", "moe_dev_upload", "moe_dev_download",
     "moe_dev_memset", "moe_dev_sync", "moe_dev_count", "moe_time_forward", "moe_time_forward_each",
+    "moe_yardstick_mfma", "moe_yardstick_hbm",
 ]
 
 
@@ -67,6 +68,7 @@ def lib() -> C.CDLL:
         L.moe_expert_gemms.argtypes = [vp, ci, vp, ci, vp]
         L.moe_combine.argtypes = [vp, vp, vp, ci, vp, ci, vp]
         L.moe_dispatch_static.argtypes = [vp, vp, ci, ci, vp, vp, vp]
+        L.moe_set_distinct_ids.argtypes = [vp, ci]
         L.moe_profile_enable.argtypes = [vp, ci]
         L.moe_profile_read.argtypes = [vp, C.POINTER(cf), C.POINTER(ci)]
         L.moe_weight_bytes.argtypes = [vp]
@@ -82,6 +84,8 @@ def lib() -> C.CDLL:
         L.moe_dev_memset.argtypes = [vp, ci, C.c_size_t]
         L.moe_time_forward.argtypes = [vp, ci, vp, vp, ci, vp, ci, ci, C.POINTER(cf)]
         L.moe_time_forward_each.argtypes = [vp, ci, vp, vp, ci, vp, ci, C.POINTER(cf)]
+        L.moe_yardstick_mfma.argtypes = [ci, ci, ci, C.POINTER(C.c_double), C.POINTER(C.c_double)]
+        L.moe_yardstick_hbm.argtypes = [C.c_size_t, ci, C.POINTER(C.c_double), C.POINTER(C.c_double)]
         _lib = L
     return _lib
 
@@ -141,6 +145,20 @@ def dispatch_static(topk_i, pos, n_tokens, n_experts, offsets, perm, stream=None
     """moe_dispatch_static: no handle, no allocation; device buffers in and out."""
     check(lib().moe_dispatch_static(_p(topk_i), _p(pos), n_tokens, n_experts, _p(offsets), _p(perm),
                                     stream))
+
+
+def yardstick_mfma(n_workgroups: int = 256, iters: int = 20000, data: bool = True):
+    """(TFLOP/s, shader GHz) of a register-resident v_mfma_f32_32x32x16_bf16 loop."""
+    tf, ghz = C.c_double(), C.c_double()
+    check(lib().moe_yardstick_mfma(n_workgroups, iters, 1 if data else 0, C.byref(tf), C.byref(ghz)))
+    return float(tf.value), float(ghz.value)
+
+
+def yardstick_hbm(nbytes: int = 1 << 30, iters: int = 10):
+    """(copy GB/s counting reads + writes, read-only GB/s) of plain streams over nbytes."""
+    c, r = C.c_double(), C.c_double()
+    check(lib().moe_yardstick_hbm(nbytes, iters, C.byref(c), C.byref(r)))
+    return float(c.value), float(r.value)
 
 
 def sync() -> None:
@@ -219,6 +237,9 @@ class Moe:
     def combine(self, topk_v, pos, n_tokens, out, accumulate=False, stream=None):
         check(lib().moe_combine(self.h, _p(topk_v), _p(pos), n_tokens, _p(out),
                                 1 if accumulate else 0, stream))
+
+    def set_distinct_ids(self, distinct=True):
+        check(lib().moe_set_distinct_ids(self.h, 1 if distinct else 0))
 
     def profile_enable(self, n_calls):
         check(lib().moe_profile_enable(self.h, n_calls))

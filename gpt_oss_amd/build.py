@@ -8,7 +8,7 @@ import sys
 PKG = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(PKG, "csrc")
 LIB = os.path.join(PKG, "libmi355_moe.so")
-SOURCES = ["moe_api.hip", "pack.hip", "router.hip", "dispatch.hip", "gemm.hip", "norm.hip"]
+SOURCES = ["moe_api.hip", "pack.hip", "router.hip", "dispatch.hip", "gemm.hip", "norm.hip", "yardstick.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",

@@ -454,7 +454,7 @@ __global__ __launch_bounds__(256) void combine_kernel(const float *__restrict__ 
                                                      const int *__restrict__ inv,
                                                      const float *__restrict__ topk_v,
                                                      const int *__restrict__ pos, void *outp, int H,
-                                                     int accumulate, DirectIds ids) {
+                                                     int ldy, int accumulate, DirectIds ids) {
   const int t = blockIdx.x;
   const bool active = !(pos && pos[t] < 0);
   if (!active && (accumulate || RESID)) return;
@@ -494,7 +494,7 @@ __global__ __launch_bounds__(256) void combine_kernel(const float *__restrict__ 
 #pragma unroll
     for (int k = 0; k < kTopK; k++) {
       if (p[k] >= 0) {
-        const float4 v = reinterpret_cast<const float4 *>(y + (size_t)p[k] * H)[c];
+        const float4 v = reinterpret_cast<const float4 *>(y + (size_t)p[k] * ldy)[c];
         s.x += w[k] * v.x; s.y += w[k] * v.y; s.z += w[k] * v.z; s.w += w[k] * v.w;
       }
     }
@@ -541,24 +541,24 @@ hipError_t launch_dispatch(const int *topk_i, const int *pos, int T, int E, int 
   return hipGetLastError();
 }
 
-hipError_t launch_combine(const float *y, const int *inv, const float *topk_v, const int *pos,
+hipError_t launch_combine(const float *y, int ldy, const int *inv, const float *topk_v, const int *pos,
                           float *out, int T, int H, int accumulate, const DirectIds &direct,
                           hipStream_t s) {
   if (direct.topk_i) {
-    combine_kernel<false, true><<<T, 256, 0, s>>>(y, inv, topk_v, pos, out, H, accumulate, direct);
+    combine_kernel<false, true><<<T, 256, 0, s>>>(y, inv, topk_v, pos, out, H, ldy, accumulate, direct);
   } else {
-    combine_kernel<false, false><<<T, 256, 0, s>>>(y, inv, topk_v, pos, out, H, accumulate, direct);
+    combine_kernel<false, false><<<T, 256, 0, s>>>(y, inv, topk_v, pos, out, H, ldy, accumulate, direct);
   }
   return hipGetLastError();
 }
 
-hipError_t launch_combine_residual(const float *y, const int *inv, const float *topk_v,
+hipError_t launch_combine_residual(const float *y, int ldy, const int *inv, const float *topk_v,
                                    const int *pos, uint16_t *x, int T, int H, const DirectIds &direct,
                                    hipStream_t s) {
   if (direct.topk_i) {
-    combine_kernel<true, true><<<T, 256, 0, s>>>(y, inv, topk_v, pos, x, H, 0, direct);
+    combine_kernel<true, true><<<T, 256, 0, s>>>(y, inv, topk_v, pos, x, H, ldy, 0, direct);
   } else {
-    combine_kernel<true, false><<<T, 256, 0, s>>>(y, inv, topk_v, pos, x, H, 0, direct);
+    combine_kernel<true, false><<<T, 256, 0, s>>>(y, inv, topk_v, pos, x, H, ldy, 0, direct);
   }
   return hipGetLastError();
 }

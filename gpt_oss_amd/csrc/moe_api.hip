@@ -52,6 +52,7 @@ struct moe_handle {
   moe_config cfg{};
   int device = 0;
   int E_pad = 0;
+  int Hp = 0, IMp = 0;  // hidden / inter as the GEMMs see them: padded to multiples of 64
   std::vector<LayerWeights> layers;
   size_t layer_bytes = 0;
   size_t ws_bytes = 0;
@@ -65,6 +66,8 @@ struct moe_handle {
   int a_pad_cap = 0;  // max padded rows
   int n_blk_cap = 0;
   int disp_tokens = -1;  // batch of the last moe_dispatch (stage-level calls), -1: none
+  bool gemms_done = false;  // moe_expert_gemms has run on that dispatch: y holds its rows
+  bool distinct_ids = false;  // moe_set_distinct_ids: caller-supplied ids name an expert once per token
   // The last call ran without a dispatch pass (at most 64 tokens): its ids, for a
   // moe_get_dispatch that asks for the plan afterwards.  topk_i == nullptr: none.
   DirectIds unplanned{nullptr, nullptr, 0, 0};
@@ -72,6 +75,7 @@ struct moe_handle {
   uint16_t *act = nullptr;  // SwiGLU output, bf16 fragments
   float *y = nullptr;       // down output [a_pad_cap, H]
   uint16_t *t_norm = nullptr;  // normalised rows of moe_block_forward [max_tokens, H], allocated on first use
+  uint16_t *x_pad = nullptr;   // the batch's rows widened to Hp columns [max_tokens, Hp]; only where Hp != H
 
   // profiling
   std::vector<hipEvent_t> events;  // kMaxProfileCalls * (MOE_NUM_STAGES + 1)
@@ -129,11 +133,11 @@ struct StageTimer {
 };
 
 // column tiles of the two grouped GEMMs (tiles are kGemmTileNb blocks of 32 columns wide)
-inline int gate_up_col_tiles(const moe_config &c) {
-  return (2 * c.inter / kRowBlock + kGemmTileNb - 1) / kGemmTileNb;
+inline int gate_up_col_tiles(const moe_handle *h) {
+  return (2 * h->IMp / kRowBlock + kGemmTileNb - 1) / kGemmTileNb;
 }
-inline int down_col_tiles(const moe_config &c) {
-  return (c.hidden / kRowBlock + kGemmTileNb - 1) / kGemmTileNb;
+inline int down_col_tiles(const moe_handle *h) {
+  return (h->Hp / kRowBlock + kGemmTileNb - 1) / kGemmTileNb;
 }
 
 // Stages 3-4 on the plan of the last dispatch: gate_up GEMM with the SwiGLU (it
@@ -147,11 +151,15 @@ int run_gemms(moe_handle *h, int layer, const uint16_t *x, int T, int max_rows, 
   const int A = T * kTopK;
   const int mt_cap = A / kTileRows + c.experts;
   HIP_TRY(tm.mark(MOE_STAGE_GATE_UP));
+  if (h->Hp != c.hidden) {  // a hidden size that is not a multiple of 64: rows widened with zeros
+    HIP_TRY(launch_pad_rows(x, h->x_pad, T, c.hidden, h->Hp, s));
+    x = h->x_pad;
+  }
   HIP_TRY(launch_gate_up(x, lw.w1q ? static_cast<const void *>(lw.w1q) : lw.w1, lw.w1s, lw.b1g, lw.b1u,
-                         h->disp, h->act, c.hidden, c.inter, c.swiglu_limit, mt_cap, max_rows, direct, s));
+                         h->disp, h->act, h->Hp, h->IMp, c.swiglu_limit, mt_cap, max_rows, direct, s));
   HIP_TRY(tm.mark(MOE_STAGE_DOWN));
   HIP_TRY(launch_down(h->act, lw.w2q ? static_cast<const void *>(lw.w2q) : lw.w2, lw.w2s, lw.b2,
-                      h->disp, h->y, c.hidden, c.inter, mt_cap, max_rows, direct, s));
+                      h->disp, h->y, h->Hp, h->IMp, mt_cap, max_rows, direct, s));
   return MOE_OK;
 }
 
@@ -161,9 +169,9 @@ int run_combine(moe_handle *h, const float *topk_v, const int *pos, int T, float
                 uint16_t *resid, const DirectIds &direct, hipStream_t s, StageTimer &tm) {
   HIP_TRY(tm.mark(MOE_STAGE_COMBINE));
   if (out) {
-    HIP_TRY(launch_combine(h->y, h->disp.inv, topk_v, pos, out, T, h->cfg.hidden, accumulate, direct, s));
+    HIP_TRY(launch_combine(h->y, h->Hp, h->disp.inv, topk_v, pos, out, T, h->cfg.hidden, accumulate, direct, s));
   } else {
-    HIP_TRY(launch_combine_residual(h->y, h->disp.inv, topk_v, pos, resid, T, h->cfg.hidden, direct, s));
+    HIP_TRY(launch_combine_residual(h->y, h->Hp, h->disp.inv, topk_v, pos, resid, T, h->cfg.hidden, direct, s));
   }
   HIP_TRY(tm.mark(MOE_NUM_STAGES));
   return MOE_OK;
@@ -180,9 +188,10 @@ int run_experts(moe_handle *h, int layer, const uint16_t *x, const int *pos, con
   const bool direct_plan = direct_plan_fits(T, max_rows, c.experts, h->a_pad_cap);
   const DirectIds direct{direct_plan ? topk_i : nullptr, pos, T, c.experts};
   if (!direct_plan)
-    HIP_TRY(launch_dispatch(topk_i, pos, T, c.experts, gate_up_col_tiles(c), down_col_tiles(c), h->disp, s));
+    HIP_TRY(launch_dispatch(topk_i, pos, T, c.experts, gate_up_col_tiles(h), down_col_tiles(h), h->disp, s));
   h->unplanned = direct;
   h->disp_tokens = -1;  // the plan now belongs to this call, not to a moe_dispatch
+  h->gemms_done = false;
   int rc = run_gemms(h, layer, x, T, max_rows, direct, s, tm);
   if (rc != MOE_OK) return rc;
   return run_combine(h, topk_v, pos, T, out, accumulate, resid, direct, s, tm);
@@ -200,8 +209,8 @@ int moe_create(const moe_config *cfg, moe_handle **out) {
   *out = nullptr;
   if (cfg->topk != kTopK)
     return fail(MOE_ERR_UNSUPPORTED, "topk %d unsupported (kernels are built for 4)", cfg->topk);
-  if (cfg->hidden <= 0 || cfg->hidden % 64 || cfg->inter <= 0 || cfg->inter % 64)
-    return fail(MOE_ERR_UNSUPPORTED, "hidden %d / inter %d must be positive multiples of 64",
+  if (cfg->hidden <= 0 || cfg->hidden % 32 || cfg->inter <= 0 || cfg->inter % 32)
+    return fail(MOE_ERR_UNSUPPORTED, "hidden %d / inter %d must be positive multiples of 32",
                 cfg->hidden, cfg->inter);
   if (cfg->experts < kTopK || cfg->experts > 256)
     return fail(MOE_ERR_UNSUPPORTED, "experts %d outside [4,256]", cfg->experts);
@@ -216,6 +225,8 @@ int moe_create(const moe_config *cfg, moe_handle **out) {
   if (!h) return fail(MOE_ERR_BAD_ARG, "out of host memory");
   h->cfg = *cfg;
   h->E_pad = next_router_pad(cfg->experts);
+  h->Hp = padded_dim(cfg->hidden);
+  h->IMp = padded_dim(cfg->inter);
   hipError_t e = hipGetDevice(&h->device);
   if (e != hipSuccess) {
     delete h;
@@ -243,13 +254,14 @@ int moe_create(const moe_config *cfg, moe_handle **out) {
   ALLOC(h->disp.totals, (size_t)kTotInts);
   {
     const int mt_cap = h->a_cap / kTileRows + E;  // row tiles at max_tokens, at most
-    h->disp.tile_cap_gate_up = mt_cap * gate_up_col_tiles(*cfg);
-    h->disp.tile_cap_down = mt_cap * down_col_tiles(*cfg);
+    h->disp.tile_cap_gate_up = mt_cap * gate_up_col_tiles(h);
+    h->disp.tile_cap_down = mt_cap * down_col_tiles(h);
   }
   ALLOC(h->disp.tiles_gate_up, (size_t)h->disp.tile_cap_gate_up);
   ALLOC(h->disp.tiles_down, (size_t)h->disp.tile_cap_down);
-  ALLOC(h->act, (size_t)h->a_pad_cap * IM);
-  ALLOC(h->y, (size_t)h->a_pad_cap * H);
+  ALLOC(h->act, (size_t)h->a_pad_cap * h->IMp);
+  ALLOC(h->y, (size_t)h->a_pad_cap * h->Hp);
+  if (h->Hp != H) ALLOC(h->x_pad, (size_t)T * h->Hp);
 #undef ALLOC
   h->disp.a_pad_cap = h->a_pad_cap;
   if (rc != MOE_OK) {
@@ -257,8 +269,8 @@ int moe_create(const moe_config *cfg, moe_handle **out) {
     return rc;
   }
   h->layer_bytes = (size_t)h->E_pad * H * 2 + (size_t)h->E_pad * 4 +
-                   (size_t)E * 2 * IM * H * 2 + (size_t)E * 2 * IM * 4 +
-                   (size_t)E * H * IM * 2 + (size_t)E * H * 4;
+                   (size_t)E * 2 * h->IMp * h->Hp * 2 + (size_t)E * 2 * h->IMp * 4 +
+                   (size_t)E * h->Hp * h->IMp * 2 + (size_t)E * h->Hp * 4;
   *out = h;
   return MOE_OK;
 }
@@ -274,7 +286,7 @@ int moe_destroy(moe_handle *h) {
   (void)hipFree(h->disp.blk_counts); (void)hipFree(h->disp.offsets); (void)hipFree(h->disp.perm);
   (void)hipFree(h->disp.rowmap); (void)hipFree(h->disp.inv); (void)hipFree(h->disp.info); (void)hipFree(h->disp.totals);
   (void)hipFree(h->disp.tiles_gate_up); (void)hipFree(h->disp.tiles_down);
-  (void)hipFree(h->act); (void)hipFree(h->y); (void)hipFree(h->t_norm);
+  (void)hipFree(h->act); (void)hipFree(h->y); (void)hipFree(h->t_norm); (void)hipFree(h->x_pad);
   for (hipEvent_t ev : h->events) (void)hipEventDestroy(ev);
   delete h;
   return MOE_OK;
@@ -293,6 +305,7 @@ struct ExpertSource {
 int upload_layer(moe_handle *h, int layer, const float *w_router, const float *b_router,
                  const float *b_mlp1, const float *b_mlp2, const ExpertSource &src) {
   const int E = h->cfg.experts, H = h->cfg.hidden, IM = h->cfg.inter, E_pad = h->E_pad;
+  const int Hp = h->Hp, IMp = h->IMp;
   LayerWeights &lw = h->layers[layer];
   // not usable until this upload has gone through: a failure below leaves the
   // layer without weights rather than with freed or half-written ones
@@ -304,6 +317,7 @@ int upload_layer(moe_handle *h, int layer, const float *w_router, const float *b
   // GEMMs decode them in registers.
   const bool keep_fp4 = src.mxfp4;
   const size_t n1 = (size_t)2 * IM * H, n2 = (size_t)H * IM;  // elements of one expert's matrices
+  const size_t p1 = (size_t)2 * IMp * Hp, p2 = (size_t)Hp * IMp;  // ... as packed (sides padded to 64)
   // a layer uploaded again in the other format gives the old copy back
   if (keep_fp4) {
     (void)hipFree(lw.w1); (void)hipFree(lw.w2);
@@ -315,17 +329,17 @@ int upload_layer(moe_handle *h, int layer, const float *w_router, const float *b
   }
   ALLOCW(lw.wr, (size_t)E_pad * H);
   ALLOCW(lw.br, (size_t)E_pad + 2);
-  ALLOCW(lw.b1g, (size_t)E * IM);
-  ALLOCW(lw.b1u, (size_t)E * IM);
-  ALLOCW(lw.b2, (size_t)E * H);
+  ALLOCW(lw.b1g, (size_t)E * IMp);
+  ALLOCW(lw.b1u, (size_t)E * IMp);
+  ALLOCW(lw.b2, (size_t)E * Hp);
   if (keep_fp4) {
-    ALLOCW(lw.w1q, (size_t)E * n1 / 2);
-    ALLOCW(lw.w1s, (size_t)E * n1 / 64);  // two scale bytes per uint16
-    ALLOCW(lw.w2q, (size_t)E * n2 / 2);
-    ALLOCW(lw.w2s, (size_t)E * n2 / 64);
+    ALLOCW(lw.w1q, (size_t)E * p1 / 2);
+    ALLOCW(lw.w1s, (size_t)E * p1 / 64);  // two scale bytes per uint16
+    ALLOCW(lw.w2q, (size_t)E * p2 / 2);
+    ALLOCW(lw.w2s, (size_t)E * p2 / 64);
   } else {
-    ALLOCW(lw.w1, (size_t)E * n1);
-    ALLOCW(lw.w2, (size_t)E * n2);
+    ALLOCW(lw.w1, (size_t)E * p1);
+    ALLOCW(lw.w2, (size_t)E * p2);
   }
 #undef ALLOCW
   if (rc != MOE_OK) return rc;
@@ -348,10 +362,10 @@ int upload_layer(moe_handle *h, int layer, const float *w_router, const float *b
     HIP_TRY(launch_router_stats(stage, stage_b, E, H, lw.br + E_pad, nullptr));
     HIP_TRY(hipDeviceSynchronize());
     HIP_TRY(hipMemcpy(stage_b, b_mlp1, (size_t)E * 2 * IM * sizeof(float), hipMemcpyHostToDevice));
-    HIP_TRY(launch_pack_bias(stage_b, lw.b1g, lw.b1u, E * 2 * IM, true, nullptr));
+    HIP_TRY(launch_pack_bias(stage_b, lw.b1g, lw.b1u, E, 2 * IM, 2 * IMp, true, nullptr));
     HIP_TRY(hipDeviceSynchronize());
     HIP_TRY(hipMemcpy(stage_b, b_mlp2, (size_t)E * H * sizeof(float), hipMemcpyHostToDevice));
-    HIP_TRY(launch_pack_bias(stage_b, lw.b2, nullptr, E * H, false, nullptr));
+    HIP_TRY(launch_pack_bias(stage_b, lw.b2, nullptr, E, H, Hp, false, nullptr));
     HIP_TRY(hipDeviceSynchronize());
     // the staging buffer holds either an fp32 matrix or, in its place, the
     // (eight times smaller) blocks followed by the scales of an MXFP4 matrix
@@ -359,23 +373,23 @@ int upload_layer(moe_handle *h, int layer, const float *w_router, const float *b
     for (int ex = 0; ex < E; ex++) {
       if (!src.mxfp4) {
         HIP_TRY(hipMemcpy(stage, src.w1 + ex * n1, n1 * sizeof(float), hipMemcpyHostToDevice));
-        HIP_TRY(launch_pack_weight(stage, lw.w1 + ex * n1, 2 * IM, H, true, nullptr));
+        HIP_TRY(launch_pack_weight(stage, lw.w1 + ex * p1, 2 * IM, H, 2 * IMp, Hp, true, nullptr));
         HIP_TRY(hipDeviceSynchronize());
         HIP_TRY(hipMemcpy(stage, src.w2 + ex * n2, n2 * sizeof(float), hipMemcpyHostToDevice));
-        HIP_TRY(launch_pack_weight(stage, lw.w2 + ex * n2, H, IM, false, nullptr));
+        HIP_TRY(launch_pack_weight(stage, lw.w2 + ex * p2, H, IM, Hp, IMp, false, nullptr));
         HIP_TRY(hipDeviceSynchronize());
       } else {
         HIP_TRY(hipMemcpy(stage_u8, src.w1_blocks + ex * (n1 / 2), n1 / 2, hipMemcpyHostToDevice));
         HIP_TRY(hipMemcpy(stage_u8 + n1 / 2, src.w1_scales + ex * (n1 / 32), n1 / 32,
                           hipMemcpyHostToDevice));
-        HIP_TRY(launch_pack_fp4(stage_u8, stage_u8 + n1 / 2, lw.w1q + ex * (n1 / 2),
-                                lw.w1s + ex * (n1 / 64), 2 * IM, H, true, nullptr));
+        HIP_TRY(launch_pack_fp4(stage_u8, stage_u8 + n1 / 2, lw.w1q + ex * (p1 / 2),
+                                lw.w1s + ex * (p1 / 64), 2 * IM, H, 2 * IMp, Hp, true, nullptr));
         HIP_TRY(hipDeviceSynchronize());
         HIP_TRY(hipMemcpy(stage_u8, src.w2_blocks + ex * (n2 / 2), n2 / 2, hipMemcpyHostToDevice));
         HIP_TRY(hipMemcpy(stage_u8 + n2 / 2, src.w2_scales + ex * (n2 / 32), n2 / 32,
                           hipMemcpyHostToDevice));
-        HIP_TRY(launch_pack_fp4(stage_u8, stage_u8 + n2 / 2, lw.w2q + ex * (n2 / 2),
-                                lw.w2s + ex * (n2 / 64), H, IM, false, nullptr));
+        HIP_TRY(launch_pack_fp4(stage_u8, stage_u8 + n2 / 2, lw.w2q + ex * (p2 / 2),
+                                lw.w2s + ex * (p2 / 64), H, IM, Hp, IMp, false, nullptr));
         HIP_TRY(hipDeviceSynchronize());
       }
     }
@@ -446,9 +460,10 @@ int moe_dispatch(moe_handle *h, const int *topk_i, const int *pos, int n_tokens,
   if (n_tokens > h->cfg.max_tokens)
     return fail(MOE_ERR_CAPACITY, "n_tokens %d exceeds max_tokens %d", n_tokens, h->cfg.max_tokens);
   if (n_tokens > 0 && !topk_i) return fail(MOE_ERR_BAD_ARG, "null device pointer");
-  HIP_TRY(launch_dispatch(topk_i, pos, n_tokens, h->cfg.experts, gate_up_col_tiles(h->cfg),
-                          down_col_tiles(h->cfg), h->disp, static_cast<hipStream_t>(stream)));
+  HIP_TRY(launch_dispatch(topk_i, pos, n_tokens, h->cfg.experts, gate_up_col_tiles(h),
+                          down_col_tiles(h), h->disp, static_cast<hipStream_t>(stream)));
   h->disp_tokens = n_tokens;
+  h->gemms_done = false;
   h->unplanned.topk_i = nullptr;
   return MOE_OK;
 }
@@ -461,7 +476,7 @@ int moe_get_dispatch(moe_handle *h, int *offsets, int *perm, int n_tokens, void 
   if (h->unplanned.topk_i) {
     const moe_config &c = h->cfg;
     HIP_TRY(launch_dispatch(h->unplanned.topk_i, h->unplanned.pos, h->unplanned.T, c.experts,
-                            gate_up_col_tiles(c), down_col_tiles(c), h->disp, s));
+                            gate_up_col_tiles(h), down_col_tiles(h), h->disp, s));
     h->unplanned.topk_i = nullptr;
   }
   if (offsets)
@@ -482,8 +497,10 @@ int moe_experts(moe_handle *h, int layer, const uint16_t *x, const int *pos, con
   hipStream_t s = static_cast<hipStream_t>(stream);
   StageTimer tm(h, s);
   HIP_TRY(tm.mark(MOE_STAGE_ROUTER));
-  // ids from outside may name an expert in several slots of a token
-  rc = run_experts(h, layer, x, pos, topk_i, topk_v, n_tokens, n_tokens * kTopK, out, accumulate, s, tm);
+  // ids from outside may name an expert in several slots of a token, unless the
+  // caller has said otherwise (moe_set_distinct_ids)
+  const int max_rows = h->distinct_ids ? n_tokens : n_tokens * kTopK;
+  rc = run_experts(h, layer, x, pos, topk_i, topk_v, n_tokens, max_rows, out, accumulate, s, tm);
   if (rc == MOE_OK) tm.done();
   return rc;
 }
@@ -499,7 +516,10 @@ int moe_expert_gemms(moe_handle *h, int layer, const uint16_t *x, int n_tokens, 
   StageTimer tm(h, nullptr);  // stage-level calls are not timed
   tm.ev = nullptr;
   // the ids of a moe_dispatch come from outside and may name an expert in several slots of a token
-  return run_gemms(h, layer, x, n_tokens, n_tokens * kTopK, DirectIds{nullptr, nullptr, 0, 0}, s, tm);
+  const int max_rows = h->distinct_ids ? n_tokens : n_tokens * kTopK;
+  rc = run_gemms(h, layer, x, n_tokens, max_rows, DirectIds{nullptr, nullptr, 0, 0}, s, tm);
+  if (rc == MOE_OK) h->gemms_done = true;
+  return rc;
 }
 
 int moe_combine(moe_handle *h, const float *topk_v, const int *pos, int n_tokens, float *out,
@@ -510,6 +530,8 @@ int moe_combine(moe_handle *h, const float *topk_v, const int *pos, int n_tokens
     return fail(MOE_ERR_STATE, "moe_combine(%d tokens) needs moe_dispatch and moe_expert_gemms of the same batch first (last: %d)",
                 n_tokens, h->disp_tokens);
   if (n_tokens == 0) return MOE_OK;
+  if (!h->gemms_done)
+    return fail(MOE_ERR_STATE, "moe_combine(%d tokens): moe_expert_gemms has not run on this dispatch", n_tokens);
   if (!topk_v || !out) return fail(MOE_ERR_BAD_ARG, "null device pointer");
   StageTimer tm(h, nullptr);
   tm.ev = nullptr;
@@ -533,6 +555,12 @@ int moe_forward(moe_handle *h, int layer, const uint16_t *x, const int *pos, int
   return rc;
 }
 
+int moe_set_distinct_ids(moe_handle *h, int distinct) {
+  if (!h) return fail(MOE_ERR_BAD_ARG, "null handle");
+  h->distinct_ids = distinct != 0;
+  return MOE_OK;
+}
+
 int moe_upload_norm(moe_handle *h, int layer, const float *rms_ffn_w) {
   const int rc0 = check_upload_args(h, layer);
   if (rc0 != MOE_OK) return rc0;
@@ -547,7 +575,7 @@ int moe_upload_norm(moe_handle *h, int layer, const float *rms_ffn_w) {
   HIP_TRY(hipMalloc(reinterpret_cast<void **>(&stage), (size_t)H * sizeof(float)));
   auto body = [&]() -> int {
     HIP_TRY(hipMemcpy(stage, rms_ffn_w, (size_t)H * sizeof(float), hipMemcpyHostToDevice));
-    HIP_TRY(launch_pack_bias(stage, lw.rms_w, nullptr, H, false, nullptr));  // rounds to bf16 values
+    HIP_TRY(launch_pack_bias(stage, lw.rms_w, nullptr, 1, H, H, false, nullptr));  // rounds to bf16 values
     HIP_TRY(hipDeviceSynchronize());
     return MOE_OK;
   };

@@ -100,12 +100,22 @@ struct LayerWeights {
 
 hipError_t launch_pack_router(const float *w_src, const float *b_src, uint16_t *wr, float *br,
                               int E, int E_pad, int H, hipStream_t s);
-hipError_t launch_pack_weight(const float *src, uint16_t *dst, int rows, int cols, bool gate_up,
-                              hipStream_t s);
+// The grouped GEMMs work on matrices whose sides are multiples of 64 (a double
+// step of the reduction, a pair of column blocks).  Sizes that are multiples of
+// 32 only are padded to that inside the library: zero weights and biases at
+// upload, zero columns of the routed rows per call (launch_pad_rows).  The
+// reference pads its packed weights likewise (utility/utility.cpp:558-622).
+constexpr int kDimGran = 64;
+inline int padded_dim(int n) { return (n + kDimGran - 1) / kDimGran * kDimGran; }
+// rows x cols (source) -> rows_p x cols_p (packed, zero outside the source)
+hipError_t launch_pack_weight(const float *src, uint16_t *dst, int rows, int cols, int rows_p, int cols_p,
+                              bool gate_up, hipStream_t s);
 hipError_t launch_pack_fp4(const uint8_t *blocks, const uint8_t *scales, uint8_t *wq, uint16_t *ws,
-                           int rows, int cols, bool gate_up, hipStream_t s);
-hipError_t launch_pack_bias(const float *src, float *dst_a, float *dst_b, int n, bool deinterleave,
-                            hipStream_t s);
+                           int rows, int cols, int rows_p, int cols_p, bool gate_up, hipStream_t s);
+// n_rows rows of len values -> rows of len_p (each half len_p / 2 when de-interleaving)
+hipError_t launch_pack_bias(const float *src, float *dst_a, float *dst_b, int n_rows, int len, int len_p,
+                            bool deinterleave, hipStream_t s);
+hipError_t launch_pad_rows(const uint16_t *x, uint16_t *xp, int T, int H, int Hp, hipStream_t s);
 
 // rstat: two floats written by launch_router_stats at upload (largest 2-norm of
 // an expert's router weights, largest bias magnitude), the inputs of the error
@@ -170,10 +180,11 @@ hipError_t launch_down(const uint16_t *act, const void *w2, const uint16_t *w2_s
                        const DispatchBuffers &d, float *y, int H, int IM, int mt_cap, int max_rows,
                        const DirectIds &direct, hipStream_t s);
 // direct.topk_i != nullptr: the rows of y are found from the ids (inv is not read)
-hipError_t launch_combine(const float *y, const int *inv, const float *topk_v, const int *pos,
+// ldy: floats per row of y (the padded hidden size)
+hipError_t launch_combine(const float *y, int ldy, const int *inv, const float *topk_v, const int *pos,
                           float *out, int T, int H, int accumulate, const DirectIds &direct,
                           hipStream_t s);
-hipError_t launch_combine_residual(const float *y, const int *inv, const float *topk_v,
+hipError_t launch_combine_residual(const float *y, int ldy, const int *inv, const float *topk_v,
                                    const int *pos, uint16_t *x, int T, int H, const DirectIds &direct,
                                    hipStream_t s);
 hipError_t launch_rmsnorm(const uint16_t *x, const float *weight, const int *pos, uint16_t *t_out,

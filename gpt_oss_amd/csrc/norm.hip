@@ -59,6 +59,28 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(const uint16_t *__restrict
   }
 }
 
+// Rows of H bf16 values copied into rows of Hp >= H, the rest zero: the grouped
+// GEMMs reduce over multiples of 64, and a hidden size that is not one (the
+// reference's 7M model has 32, export_model_bin/gpt-oss-7m/config.json:3) is
+// widened here, once per call, rather than read past the end of its rows.
+__global__ __launch_bounds__(256) void pad_rows_kernel(const uint4 *__restrict__ x, uint4 *__restrict__ xp,
+                                                      int T, int H8, int Hp8) {
+  const size_t n = (size_t)T * Hp8;
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256) {
+    const size_t t = i / Hp8;
+    const int c = (int)(i % Hp8);
+    xp[i] = c < H8 ? x[t * H8 + c] : make_uint4(0u, 0u, 0u, 0u);
+  }
+}
+
+hipError_t launch_pad_rows(const uint16_t *x, uint16_t *xp, int T, int H, int Hp, hipStream_t s) {
+  const size_t n = (size_t)T * (Hp / 8);
+  const int grid = (int)((n + 255) / 256 < 4096 ? (n + 255) / 256 : 4096);
+  pad_rows_kernel<<<grid, 256, 0, s>>>(reinterpret_cast<const uint4 *>(x), reinterpret_cast<uint4 *>(xp), T,
+                                       H / 8, Hp / 8);
+  return hipGetLastError();
+}
+
 hipError_t launch_rmsnorm(const uint16_t *x, const float *weight, const int *pos, uint16_t *t_out,
                           int T, int H, hipStream_t s) {
   rmsnorm_kernel<<<(T + 3) / 4, 256, 0, s>>>(x, weight, pos, t_out, T, H);

@@ -18,10 +18,14 @@ __device__ __forceinline__ float bf16_round(float f) {
 // (source rows 2j) and row block 2p+1 the up rows (source rows 2j+1) of
 // j = 32p .. 32p+31, so that a lane's gate and up accumulators line up and the
 // SwiGLU epilogue needs no exchange between lanes.
+//
+// The packed matrix has rows_p x cols_p elements (multiples of 64, see
+// padded_dim); what lies outside the source's rows x cols is zero, so that a
+// padded reduction adds nothing and a padded output column is its bias alone.
 __global__ void pack_weight_kernel(const float *__restrict__ src, uint4 *__restrict__ dst, int rows,
-                                   int cols, int gate_up) {
-  const int kb_total = cols / kFragK;
-  const size_t n_chunks = (size_t)(rows / kRowBlock) * kb_total * 64;
+                                   int cols, int rows_p, int cols_p, int gate_up) {
+  const int kb_total = cols_p / kFragK;
+  const size_t n_chunks = (size_t)(rows_p / kRowBlock) * kb_total * 64;
   for (size_t c = (size_t)blockIdx.x * blockDim.x + threadIdx.x; c < n_chunks;
        c += (size_t)gridDim.x * blockDim.x) {
     const int lane = (int)(c & 63);
@@ -31,9 +35,13 @@ __global__ void pack_weight_kernel(const float *__restrict__ src, uint4 *__restr
     const int n = lane & 31;
     const int k0 = kb * kFragK + 8 * (lane >> 5);
     const int row = gate_up ? 2 * (kRowBlock * (nb >> 1) + n) + (nb & 1) : kRowBlock * nb + n;
+    uint4 o = make_uint4(0u, 0u, 0u, 0u);
+    if (row >= rows || k0 >= cols) {  // cols is a multiple of 8: a piece lies inside or outside
+      dst[c] = o;
+      continue;
+    }
     const float4 *p = reinterpret_cast<const float4 *>(src + (size_t)row * cols + k0);
     const float4 a = p[0], b = p[1];
-    uint4 o;
     o.x = f32_to_bf16_rne(a.x) | ((uint32_t)f32_to_bf16_rne(a.y) << 16);
     o.y = f32_to_bf16_rne(a.z) | ((uint32_t)f32_to_bf16_rne(a.w) << 16);
     o.z = f32_to_bf16_rne(b.x) | ((uint32_t)f32_to_bf16_rne(b.y) << 16);
@@ -55,11 +63,13 @@ __global__ void pack_weight_kernel(const float *__restrict__ src, uint4 *__restr
 //   bytes 8-15  the same for block 2P+1,
 // and for every n the two scale bytes (block 2P, block 2P+1).  With gate_up set
 // the row blocks are the (gate, up) pairs of pack_weight_kernel.
+// Rows and steps of the padded matrix (rows_p x cols_p) outside the source are
+// zero nibbles with scale byte 127 (2^0).
 __global__ void pack_fp4_kernel(const uint8_t *__restrict__ blocks, const uint8_t *__restrict__ scales,
                                 uint4 *__restrict__ wq, uint16_t *__restrict__ ws, int rows, int cols,
-                                int gate_up) {
-  const int steps = cols / 32;
-  const int pairs = rows / (2 * kRowBlock);
+                                int rows_p, int cols_p, int gate_up) {
+  const int steps = cols_p / 32, src_steps = cols / 32;
+  const int pairs = rows_p / (2 * kRowBlock);
   const size_t n_chunks = (size_t)pairs * steps * 64;
   for (size_t c = (size_t)blockIdx.x * blockDim.x + threadIdx.x; c < n_chunks;
        c += (size_t)gridDim.x * blockDim.x) {
@@ -74,7 +84,12 @@ __global__ void pack_fp4_kernel(const uint8_t *__restrict__ blocks, const uint8_
     for (int j = 0; j < 2; j++) {
       const int nb = 2 * P + j;
       const int row = gate_up ? 2 * (kRowBlock * (nb >> 1) + n) + (nb & 1) : kRowBlock * nb + n;
-      const size_t g = (size_t)row * steps + step;
+      if (row >= rows || step >= src_steps) {
+        o[2 * j + 0] = o[2 * j + 1] = 0u;
+        sc |= 127u << (8 * j);
+        continue;
+      }
+      const size_t g = (size_t)row * src_steps + step;
       const uint8_t *src = blocks + g * 16;
       o[2 * j + 0] = *reinterpret_cast<const uint32_t *>(src + 4 * h);
       o[2 * j + 1] = *reinterpret_cast<const uint32_t *>(src + 8 + 4 * h);
@@ -112,13 +127,17 @@ __global__ void pack_router_kernel(const float *__restrict__ w, const float *__r
 
 // Biases are kept as fp32 holding bf16-rounded values (the reference keeps
 // them as bf16, expert.cpp:906-930).  deinterleave: src[2j] -> a[j], src[2j+1] -> b[j].
+// The source holds rows of `len` values, the destination rows of len_p >= len
+// (of len_p / 2 for each half when de-interleaving); the padding is zero.
 __global__ void pack_bias_kernel(const float *__restrict__ src, float *__restrict__ a,
-                                 float *__restrict__ b, int n, int deinterleave) {
+                                 float *__restrict__ b, int n_rows, int len, int len_p, int deinterleave) {
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
-  if (i >= n) return;
-  const float v = bf16_round(src[i]);
+  if (i >= n_rows * len_p) return;
+  const int r = i / len_p, j = i % len_p;
+  const float v = j < len ? bf16_round(src[(size_t)r * len + j]) : 0.f;
   if (deinterleave) {
-    if (i & 1) b[i >> 1] = v; else a[i >> 1] = v;
+    const size_t o = (size_t)r * (len_p / 2) + (j >> 1);
+    if (j & 1) b[o] = v; else a[o] = v;
   } else {
     a[i] = v;
   }
@@ -130,23 +149,25 @@ hipError_t launch_pack_router(const float *w_src, const float *b_src, uint16_t *
   return hipGetLastError();
 }
 
-hipError_t launch_pack_weight(const float *src, uint16_t *dst, int rows, int cols, bool gate_up,
-                              hipStream_t s) {
-  pack_weight_kernel<<<2048, 256, 0, s>>>(src, reinterpret_cast<uint4 *>(dst), rows, cols,
+hipError_t launch_pack_weight(const float *src, uint16_t *dst, int rows, int cols, int rows_p, int cols_p,
+                              bool gate_up, hipStream_t s) {
+  pack_weight_kernel<<<2048, 256, 0, s>>>(src, reinterpret_cast<uint4 *>(dst), rows, cols, rows_p, cols_p,
                                           gate_up ? 1 : 0);
   return hipGetLastError();
 }
 
 hipError_t launch_pack_fp4(const uint8_t *blocks, const uint8_t *scales, uint8_t *wq, uint16_t *ws,
-                           int rows, int cols, bool gate_up, hipStream_t s) {
+                           int rows, int cols, int rows_p, int cols_p, bool gate_up, hipStream_t s) {
   pack_fp4_kernel<<<2048, 256, 0, s>>>(blocks, scales, reinterpret_cast<uint4 *>(wq), ws, rows, cols,
-                                       gate_up ? 1 : 0);
+                                       rows_p, cols_p, gate_up ? 1 : 0);
   return hipGetLastError();
 }
 
-hipError_t launch_pack_bias(const float *src, float *dst_a, float *dst_b, int n, bool deinterleave,
-                            hipStream_t s) {
-  pack_bias_kernel<<<(n + 255) / 256, 256, 0, s>>>(src, dst_a, dst_b, n, deinterleave ? 1 : 0);
+hipError_t launch_pack_bias(const float *src, float *dst_a, float *dst_b, int n_rows, int len, int len_p,
+                            bool deinterleave, hipStream_t s) {
+  const int n = n_rows * len_p;
+  pack_bias_kernel<<<(n + 255) / 256, 256, 0, s>>>(src, dst_a, dst_b, n_rows, len, len_p,
+                                                   deinterleave ? 1 : 0);
   return hipGetLastError();
 }
 

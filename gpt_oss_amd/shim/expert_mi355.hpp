@@ -67,6 +67,8 @@ static void mi355_moe_init(DeviceContext &ctx, int device_id, Transformer *trans
   cfg.swiglu_limit = p->swiglu_limit;
   if ((size_t)device_id >= g_mi355_moe.size()) g_mi355_moe.resize(device_id + 1, nullptr);
   MI355_MOE_CHECK(moe_create(&cfg, &g_mi355_moe[device_id]));
+  // d_topk_i comes from the runner's top-k (utility/utility.cpp:273-365): K different experts per token
+  MI355_MOE_CHECK(moe_set_distinct_ids(g_mi355_moe[device_id], 1));
   const size_t E = p->n_experts, H = p->hidden_dim, IM = p->intermediate_dim;
   for (int l = 0; l < p->n_layers; l++) {
     // layer offsets of run.cpp:664-665, :687-690, :729-733

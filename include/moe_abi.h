@@ -44,8 +44,10 @@ typedef enum {
  * max_tokens replaces MAX_BATCH_SIZE / MAX_BATCH_SIZE_120B
  * (common/defines.h:30-31). */
 typedef struct {
-  int hidden;        /* H,  multiple of 64                     */
-  int inter;         /* IM, multiple of 64                     */
+  int hidden;        /* H,  multiple of 32 (padded to 64 inside, as the reference
+                        pads its packed weights, utility/utility.cpp:558-622;
+                        gpt-oss-7m has 32, export_model_bin/gpt-oss-7m/config.json:3) */
+  int inter;         /* IM, multiple of 32 (likewise)          */
   int experts;       /* E,  1..256                             */
   int topk;          /* K,  must be 4 (EXPERT_PER_TOKEN)       */
   int layers;        /* number of MoE layers held by the handle */
@@ -134,12 +136,18 @@ int moe_upload_norm(moe_handle *h, int layer, const float *rms_ffn_w);
 int moe_block_forward(moe_handle *h, int layer, uint16_t *x, const int *pos,
                       int n_tokens, void *stream);
 
-/* Stage 1 alone.  Writes topk_i int [n_tokens,K] (descending score, ties to
- * the lower expert id; -1 on inactive rows), topk_v f32 [n_tokens,K] (softmax
- * over the K selected logits) and, if score != NULL, the logits f32
+/* The router stage alone.  Writes topk_i int [n_tokens,K] (descending score,
+ * ties to the lower expert id; -1 on inactive rows), topk_v f32 [n_tokens,K]
+ * (softmax over the K selected logits) and, if score != NULL, the logits f32
  * [n_tokens,E].  Replaces matmul_router_kernel (matmul/matmul.cpp:945-1019)
  * and fused_topk_softmax_batch_kernel (utility/utility.cpp:273-365), i.e. the
- * producers of d_router_score, d_topk_i, d_topk_v (getp_run.cpp:697-716). */
+ * producers of d_router_score, d_topk_i, d_topk_v (getp_run.cpp:697-716).
+ * Accuracy: topk_i is exactly what the CPU path's arithmetic selects (float
+ * products summed in a double, run.cpp:363-369).  That arithmetic is carried
+ * out only for the logits that decide a selection; all other entries of score,
+ * and topk_v of tokens whose selection was clear from the first pass, come from
+ * a bf16 matrix-core pass with fp64 hand-over and lie within 2e-6 + 2^-22
+ * relative of the exact values. */
 int moe_router(moe_handle *h, int layer, const uint16_t *x, const int *pos,
                int n_tokens, float *score, int *topk_i, float *topk_v,
                void *stream);
@@ -163,12 +171,25 @@ int moe_dispatch(moe_handle *h, const int *topk_i, const int *pos, int n_tokens,
 int moe_get_dispatch(moe_handle *h, int *offsets, int *perm, int n_tokens,
                      void *stream);
 
-/* Stages 2-6 from caller-supplied routing: the body of
- * gpu_forward_device_batch_ep (expert.cpp:1366), which reads d_t, d_topk_i,
- * d_topk_v, d_pos and adds into d_e_agg. */
+/* Everything after the router (dispatch, both GEMMs, combine) from
+ * caller-supplied routing: the body of gpu_forward_device_batch_ep
+ * (expert.cpp:1366), which reads d_t, d_topk_i, d_topk_v, d_pos and adds into
+ * d_e_agg. */
 int moe_experts(moe_handle *h, int layer, const uint16_t *x, const int *pos,
                 const int *topk_i, const float *topk_v, int n_tokens,
                 float *out, int accumulate, void *stream);
+
+/* Promise about caller-supplied ids (moe_experts, moe_dispatch +
+ * moe_expert_gemms): distinct != 0 says that the K ids of a token name K
+ * different experts, which holds for any top-k selection, the reference's
+ * included (run.cpp:388-421, utility/utility.cpp:273-365).  No expert then gets
+ * more rows than the batch has tokens, and batches of up to 64 tokens run the
+ * small-batch kernels (no dispatch pass, several workgroups per CU) as they do
+ * under moe_forward.  Without the promise (the default) an expert may be named
+ * in all K slots of every token and only batches of up to 16 tokens take that
+ * path.  Ids that break the promise do not fault: rows beyond an expert's 64
+ * are dropped.  Has no counterpart in the reference. */
+int moe_set_distinct_ids(moe_handle *h, int distinct);
 
 /* moe_dispatch for callers that cannot allocate device memory: code under HIP
  * graph capture, tight serving loops, harnesses that forbid hipMalloc.  It has
@@ -189,15 +210,17 @@ int moe_experts(moe_handle *h, int layer, const uint16_t *x, const int *pos,
 int moe_dispatch_static(const int *topk_i, const int *pos, int n_tokens,
                         int n_experts, int *offsets, int *perm, void *stream);
 
-/* Stages 3-5 alone, on the plan of the last moe_dispatch of the same batch:
- * gathers the routed rows of x into per-expert segments, runs the gate_up
- * grouped GEMM with the clamped SwiGLU and the down grouped GEMM, and leaves one
- * fp32 row per assignment inside the handle.  Replaces the mlp1 / mlp2 launches
- * of the local path (getp_run.cpp:788-829; kernels matmul/matmul.cpp:1023-1914). */
+/* MOE_STAGE_GATE_UP and MOE_STAGE_DOWN alone, on the plan of the last
+ * moe_dispatch of the same batch: the gate_up grouped GEMM with the clamped
+ * SwiGLU, which reads the routed token rows of x itself through the plan's row
+ * map (there is no gathered copy), then the down grouped GEMM; leaves one fp32
+ * row per assignment inside the handle.  Replaces the mlp1 / mlp2 launches of
+ * the local path (getp_run.cpp:788-829; kernels matmul/matmul.cpp:1023-1914). */
 int moe_expert_gemms(moe_handle *h, int layer, const uint16_t *x, int n_tokens,
                      void *stream);
 
-/* Stage 6 alone, after moe_dispatch and moe_expert_gemms of the same batch:
+/* MOE_STAGE_COMBINE alone, after moe_dispatch and moe_expert_gemms of the same
+ * batch (MOE_ERR_STATE if either has not run since the last dispatch):
  * out[t,:] (+)= sum_k topk_v[t,k] * (row of assignment t*K+k), slots added in
  * order 0..K-1, rows with pos < 0 skipped (accumulate) or zeroed.  Replaces
  * reduce_mlp2_slots_kernel (utility/utility.cpp:701-726, launched at
@@ -246,6 +269,26 @@ int moe_time_forward(moe_handle *h, int layer, const uint16_t *x, const int *pos
 int moe_time_forward_each(moe_handle *h, int layer, const uint16_t *x,
                           const int *pos, int n_tokens, float *out, int iters,
                           float *ms_each);
+
+/* Measured denominators for the rooflines the benchmark reports (the published
+ * peaks are 2.5 PFLOP/s dense bf16 and 8 TB/s).  They take the place of the
+ * reference's tuning harness (getp-csrc/matmul/tune.cpp:1347-1595, results in
+ * matmul/log.txt), which times its GEMM kernels against each other only.  Not
+ * used by the layer; both allocate and free their own buffers and synchronise.
+ *
+ * moe_yardstick_mfma: n_workgroups workgroups of 4 waves (one per SIMD, one
+ * workgroup per CU up to the CU count) run v_mfma_f32_32x32x16_bf16 on 16
+ * independent accumulators each from registers alone, iters x 16 per wave.
+ * data != 0: pseudo-random operands of unit scale; data == 0: zeros (the clock
+ * the matrix cores sustain depends on the bits that toggle).  Returns TFLOP/s
+ * over the launch and the mean shader clock in GHz during the loop.
+ *
+ * moe_yardstick_hbm: a copy kernel and a read-only kernel over `bytes` of
+ * device memory (choose it well above the 256 MB memory-side cache), iters
+ * launches each; copy_gbs counts bytes read plus bytes written. */
+int moe_yardstick_mfma(int n_workgroups, int iters, int data, double *tflops,
+                       double *shader_ghz);
+int moe_yardstick_hbm(size_t bytes, int iters, double *copy_gbs, double *read_gbs);
 
 #ifdef __cplusplus
 }

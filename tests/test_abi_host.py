@@ -40,8 +40,8 @@ def _create(**kw):
 
 @pytest.mark.parametrize("kw,code,word", [
     (dict(topk=2), -2, "topk"),
-    (dict(hidden=100), -2, "multiples of 64"),
-    (dict(inter=2880 + 32), -2, "multiples of 64"),
+    (dict(hidden=100), -2, "multiples of 32"),
+    (dict(inter=2880 + 16), -2, "multiples of 32"),
     (dict(experts=2), -2, "experts"),
     (dict(experts=300), -2, "experts"),
     (dict(layers=0), -1, "layers"),

@@ -1,7 +1,8 @@
 """Seeded sweep over layer shapes, batch sizes and activity masks against the
 CPU oracle, through the C-ABI: expert counts that are no power of two, hidden
-sizes that leave a narrow last column tile, batch sizes on both sides of every
-size at which the library changes its plan, handles larger than the batch.
+sizes that leave a narrow last column tile or are no multiple of 64 (padded
+inside the library), batch sizes on both sides of every size at which the
+library changes its plan, handles larger than the batch.
 
 Bars as in test_gpu_parity.py: ids, offsets and permutations bit-exact; outputs
 within max-abs 2e-2 and rel-L2 1e-3 of the oracle on the same bf16 inputs."""
@@ -15,8 +16,8 @@ pytestmark = pytest.mark.gpu
 
 W = ("w_router", "b_router", "w_mlp1", "b_mlp1", "w_mlp2", "b_mlp2")
 EXPERTS = [4, 5, 8, 13, 16, 32, 33, 64, 100, 128, 200, 256]
-HIDDEN = [64, 128, 192, 320]
-INTER = [64, 128, 256]
+HIDDEN = [32, 64, 96, 128, 192, 320]
+INTER = [32, 64, 96, 128, 256]
 TOKENS = [1, 2, 15, 16, 17, 63, 64, 65, 100, 128, 129, 255, 256, 257, 300, 511, 513, 1000, 1500, 2500]
 
 

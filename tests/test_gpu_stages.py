@@ -57,6 +57,9 @@ def test_stage_entry_points_compose(T):
         m.expert_gemms(0, dx, T)
     assert e.value.code == -5
     m.dispatch(dti, dpos, T)
+    with pytest.raises(abi.MoeError) as e:  # the GEMMs have not run on this dispatch: y is stale
+        m.combine(dtv, dpos, T, dout, accumulate=False)
+    assert e.value.code == -5
     m.expert_gemms(0, dx, T)
     m.combine(dtv, dpos, T, dout, accumulate=False)
     m.combine(dtv, dpos, T, dacc, accumulate=True)
@@ -69,6 +72,109 @@ def test_stage_entry_points_compose(T):
     m.forward(0, dx, dpos, T, dout)
     with pytest.raises(abi.MoeError):
         m.combine(dtv, dpos, T, dout)
+
+
+@pytest.mark.parametrize("T", [17, 40, 64, 65])
+def test_caller_routing_with_distinct_ids(T):
+    """moe_set_distinct_ids: with the promise that a token's ids are four
+    different experts, moe_experts bounds the rows per expert by T as
+    moe_forward does and takes the small-batch kernels up to 64 tokens; without
+    it the bound is 4 T.  Same bits either way, and the bits of moe_forward."""
+    sh = synth.LayerShape("d", T, 2880, 320, 32)
+    L = bf16_layer(sh, seed=8)
+    m = make_moe(sh, L, 128)
+    pos = np.zeros(T, np.int32)
+    pos[2::5] = -1
+    base = abi.run_layer(m, 0, L["x"], pos)
+    dx = abi.DevBuf.from_numpy(synth.to_bf16_bits(L["x"]))
+    dpos = abi.DevBuf.from_numpy(pos)
+    dti, dtv = abi.DevBuf.from_numpy(base["topk_i"]), abi.DevBuf.from_numpy(base["topk_v"])
+    dout = abi.DevBuf(T * sh.hidden * 4)
+    for distinct in (False, True, False):
+        m.set_distinct_ids(distinct)
+        dout.memset(0xFF)
+        m.experts(0, dx, dpos, dti, dtv, T, dout)
+        abi.sync()
+        assert np.array_equal(dout.download((T, sh.hidden), np.float32), base["out"]), f"distinct={distinct}"
+        m.dispatch(dti, dpos, T)
+        m.expert_gemms(0, dx, T)
+        dout.memset(0xFF)
+        m.combine(dtv, dpos, T, dout)
+        abi.sync()
+        assert np.array_equal(dout.download((T, sh.hidden), np.float32), base["out"]), f"staged, distinct={distinct}"
+    # ids that break the promise must not fault: one expert in all four slots of every token
+    m.set_distinct_ids(True)
+    bad = np.full((T, 4), 3, np.int32)
+    m.experts(0, dx, None, abi.DevBuf.from_numpy(bad), dtv, T, dout)
+    abi.sync()
+
+
+def test_reference_7m_model_shape():
+    """The reference's smallest model (export_model_bin/gpt-oss-7m/config.json:
+    hidden 32, intermediate 64, 32 experts): sizes that are multiples of 32 but
+    not of 64 are padded inside the library.  Whole layer, FFN block and MXFP4
+    upload against the oracle; batches on both sides of the small-batch limit."""
+    for H, IM, E in ((32, 64, 32), (96, 96, 32), (32, 32, 8)):
+        for T in (1, 50, 64, 300, 1100):
+            sh = synth.LayerShape("7m", T, H, IM, E)
+            L = bf16_layer(sh, seed=H + T)
+            m = make_moe(sh, L, T)
+            pos = np.zeros(T, np.int32)
+            pos[1::6] = -1
+            for p in (None, pos):
+                R = abi.run_layer(m, 0, L["x"], p)
+                _, ti, _ = ob.router(L["x"], p, L["w_router"], L["b_router"], 4)
+                off, perm, _ = ob.dispatch(ti, p, E)
+                case = f"H={H} IM={IM} E={E} T={T} masked={p is not None}"
+                assert np.array_equal(R["topk_i"], ti), case
+                assert np.array_equal(R["offsets"], off) and np.array_equal(R["perm"][:off[-1]], perm), case
+                rows = np.arange(min(T, 48))
+                want = ob.moe_layer(np.ascontiguousarray(L["x"][rows]), None if p is None else np.ascontiguousarray(p[rows]),
+                                    *[L[k] for k in W], 4, sh.limit, mode=ob.ROUND_ACT_BF16 | ob.PAR_TOKENS)
+                assert np.abs(R["out"][rows] - want).max() <= 2e-2, case
+                assert np.linalg.norm(R["out"][rows] - want) <= 1e-3 * np.linalg.norm(want), case
+            # the FFN block in place on the bf16 stream
+            rng = np.random.default_rng(T)
+            rw = synth.round_bf16((1 + 0.1 * rng.standard_normal(H)).astype(np.float32))
+            m.upload_norm(0, rw)
+            dx = abi.DevBuf.from_numpy(synth.to_bf16_bits(L["x"]))
+            m.block_forward(0, dx, abi.DevBuf.from_numpy(pos), T)
+            abi.sync()
+            got = synth.from_bf16_bits(dx.download((T, H), np.uint16))
+            rows = np.arange(min(T, 32))
+            want, _ = ob.ffn_block(np.ascontiguousarray(L["x"][rows]), np.ascontiguousarray(pos[rows]), rw,
+                                   *[L[k] for k in W], 4, sh.limit, mode=ob.ROUND_ACT_BF16 | ob.PAR_TOKENS)
+            assert np.all(np.abs(got[rows] - want) <= 2e-2 + 2.0 ** -7 * np.abs(want)), f"block H={H} T={T}"
+            assert np.array_equal(got[pos < 0], L["x"][pos < 0])
+            m.close()
+    # MXFP4 upload at sizes that need padding: bit-identical to uploading the decoded matrices
+    sh = synth.LayerShape("7q", 200, 96, 96, 8)
+    x = synth.round_bf16(synth.make_activations(sh))
+    wr, br = (synth.round_bf16(a) for a in synth.make_router(sh))
+    b1k, s1, b1, b2k, s2, b2 = synth.make_experts_mxfp4(sh)
+    b1, b2 = synth.round_bf16(b1), synth.round_bf16(b2)
+    w1, w2 = ob.mxfp4_dequant(b1k, s1), ob.mxfp4_dequant(b2k, s2)
+    m4 = abi.Moe(sh.hidden, sh.inter, sh.experts, max_tokens=sh.tokens)
+    m4.upload_layer_mxfp4(0, wr, br, b1k, s1, b1, b2k, s2, b2)
+    m32 = abi.Moe(sh.hidden, sh.inter, sh.experts, max_tokens=sh.tokens)
+    m32.upload_layer(0, wr, br, w1, b1, w2, b2)
+    for T in (200, 40):
+        a, b = abi.run_layer(m4, 0, x[:T], None), abi.run_layer(m32, 0, x[:T], None)
+        assert np.array_equal(a["out"], b["out"]) and np.isfinite(a["out"]).all()
+    with pytest.raises(abi.MoeError) as e:
+        abi.Moe(48, 64, 8, max_tokens=16)  # not a multiple of 32
+    assert e.value.code == -2
+
+
+def test_yardsticks_run():
+    """The measured denominators the benchmark reports: a register-resident MFMA
+    loop and plain streams through HBM.  Sanity only: positive, below the
+    published peaks, zeros no slower than random operands."""
+    tf, ghz = abi.yardstick_mfma(256, 2000, data=True)
+    tf0, _ = abi.yardstick_mfma(256, 2000, data=False)
+    assert 200 < tf < 2600 and 0.5 < ghz < 3.0 and tf0 > 0.9 * tf
+    c, r = abi.yardstick_hbm(1 << 28, 3)
+    assert 500 < c < 8200 and 500 < r < 8200
 
 
 def test_swiglu_clamp_points():
@@ -217,7 +323,8 @@ def test_large_batches_repeat_bit_for_bit():
     (loads complete in issue order).  4096 tokens at the 20B shape run every
     tile height and both narrow last column tiles (row split 2 in gate_up, 4 in
     down); twelve calls in a row must give the same bits, with bf16 and with
-    MXFP4 weights, and so must the FFN block at 48 tokens."""
+    MXFP4 weights, so must 7168 tokens under Zipf routing (one expert with 28
+    row tiles), and so must the FFN block at 48 tokens."""
     sh = synth.CONFIGS["c2"]
     T = sh.tokens
     wr, br = (synth.round_bf16(a) for a in synth.make_router(sh))
@@ -242,6 +349,30 @@ def test_large_batches_repeat_bit_for_bit():
                 first = got
                 assert np.isfinite(got).all()
             assert np.array_equal(got, first), f"call {i}: a repeated call gave other bits"
+    # 7168 tokens with Zipf routing: up to 28 row tiles on one expert, the deepest XCD ranges
+    z = synth.CONFIGS["c3b"]
+    T3 = z.tokens
+    m4.close()
+    mz = abi.Moe(z.hidden, z.inter, z.experts, max_tokens=T3, swiglu_limit=z.limit)
+    wrz, brz = (synth.round_bf16(a) for a in synth.make_router(z))
+    w1, w2 = ob.mxfp4_dequant(b1k, s1), ob.mxfp4_dequant(b2k, s2)
+    mz.upload_layer(0, wrz, brz, w1, b1, w2, b2)
+    del w1, w2
+    xz = synth.round_bf16(synth.make_activations(z))
+    dxz = abi.DevBuf.from_numpy(synth.to_bf16_bits(xz))
+    doz = abi.DevBuf(T3 * z.hidden * 4)
+    firstz = None
+    for i in range(12):
+        doz.memset(0xFF)
+        mz.forward(0, dxz, None, T3, doz)
+        abi.sync()
+        got = doz.download((T3, z.hidden), np.float32)
+        if firstz is None:
+            firstz = got
+            assert np.isfinite(got).all()
+        assert np.array_equal(got, firstz), f"7168 tokens, Zipf routing, call {i}: other bits"
+    mz.close()
+    del firstz, got
     rw = synth.round_bf16((1 + 0.1 * np.random.default_rng(2).standard_normal(sh.hidden)).astype(np.float32))
     m16.upload_norm(0, rw)
     ref = None
