@@ -49,9 +49,17 @@ struct PlanOut {
   int tile_cap_gate_up, tile_cap_down;
 };
 
-// The tiles of expert ee in the tile sequences of both GEMMs: tile L = (expert,
-// column tile, row tile), row tile fastest.  One wave; its lanes run over the
-// expert's tiles of both GEMMs in one sweep.
+// The tiles of expert ee in the tile sequences of both GEMMs.  An expert's row
+// tiles are taken in groups of at most kRowTileGroup (sizes as even as they go);
+// tile L = (expert, group, column tile, row tile of the group), row tile fastest.
+// The 32 CUs of an XCD then run a few column tiles of one group at a time: the
+// group's rows are fetched once per generation of tiles instead of once per
+// column tile (an expert with 28 row tiles otherwise streams all its rows
+// through the 4 MB L2 for each of its 23 column tiles).  Measured at 7168 tokens
+// with Zipf routing: the gate_up GEMM's reads from beyond L2 3.78 -> 2.77 GB, the
+// down GEMM's 1.75 -> 1.51 GB, durations unchanged; experts with up to
+// kRowTileGroup row tiles (even routing at 4096 tokens) are laid out as before.
+// One wave; its lanes run over the expert's tiles of both GEMMs in one sweep.
 __device__ __forceinline__ void write_expert_tiles(int ee, int nmt, int rbe, int exe, int rowblk, int first,
                                                    int lane, int n_ct_gate_up, int n_ct_down,
                                                    const PlanOut &out) {
@@ -61,8 +69,22 @@ __device__ __forceinline__ void write_expert_tiles(int ee, int nmt, int rbe, int
     const bool g = ii >= n_up;
     const int i = g ? ii - n_up : ii;
     const int L = first * (g ? n_ct_down : n_ct_gate_up) + i;
-    const int nt = i / nmt;
-    const int mt = i - nt * nmt;
+    const int n_ct = g ? n_ct_down : n_ct_gate_up;
+    const int n_grp = (nmt + kRowTileGroup - 1) / kRowTileGroup;
+    const int gs = nmt / n_grp, gx = nmt - gs * n_grp;  // the first gx groups hold gs + 1 row tiles
+    const int big = gx * (gs + 1) * n_ct;               // tiles of those groups
+    int grp, r, gsz;
+    if (i < big) {
+      grp = i / ((gs + 1) * n_ct);
+      r = i - grp * (gs + 1) * n_ct;
+      gsz = gs + 1;
+    } else {
+      grp = gx + (i - big) / (gs * n_ct);
+      r = (i - big) - (grp - gx) * gs * n_ct;
+      gsz = gs;
+    }
+    const int nt = r / gsz;
+    const int mt = grp * gs + min(grp, gx) + (r - nt * gsz);
     TileDesc d;
     d.e = ee;
     d.nt = nt;
@@ -155,7 +177,7 @@ __device__ __forceinline__ int build_plan(int count, int E, int n_ct_gate_up, in
   }
   __syncthreads();
   // Thread (g, x): boundary x of GEMM g = first tile at which the cost so far
-  // reaches x/8 of the total.  Tile L = (expert, column tile, row tile).
+  // reaches x/8 of the total (an expert's tiles taken as equally dear: their heights differ by one block at most).
   if (e < 2 * (kXcds + 1)) {
     const int g = e / (kXcds + 1), x = e % (kXcds + 1);
     const int n_ct = g ? n_ct_down : n_ct_gate_up;

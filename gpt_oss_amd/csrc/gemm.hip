@@ -37,11 +37,11 @@
 // differently, see there).
 //
 // Tile order.  Workgroup ids are dealt round-robin to the 8 XCDs, each with
-// its own L2.  Logical tile ids are laid out (expert, column tile, row tile)
-// with the row tile fastest, and XCD x takes a contiguous range of them (see
-// dispatch_scan_kernel: about an eighth by estimated cost): the tiles an XCD
-// runs at one time share the expert's rows and a few column slabs of its
-// weights, so each weight byte leaves HBM once.  (Batches of at most 64 tokens
+// its own L2.  Logical tile ids are laid out (expert, group of up to four row
+// tiles, column tile, row tile) with the row tile fastest, and XCD x takes a
+// contiguous range of them (see build_plan and write_expert_tiles: about an
+// eighth by estimated cost): the tiles an XCD runs at one time share a few row
+// tiles of the expert and a few column slabs of its weights.  (Batches of at most 64 tokens
 // have no tile table at all: see DIRECT at the kernel.)
 #include <type_traits>
 #include <utility>

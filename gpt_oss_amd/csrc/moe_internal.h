@@ -34,12 +34,13 @@ constexpr int kTileGran = 32;   // an expert's segment of padded rows is a multi
 constexpr float kAlpha = 1.702f;  // run.cpp:709
 
 // Work split of the grouped GEMMs over the 8 XCDs (each has an L2 of its own).
-// Tiles are numbered (expert, column tile, row tile), row tile fastest; XCD x
-// takes the tiles [bounds[x], bounds[x+1]), a range of about an eighth of the
-// estimated cost.  (Cutting the last tiles of a range into smaller pieces, so
+// Tiles are numbered (expert, group of row tiles, column tile, row tile of the
+// group), row tile fastest; XCD x takes the tiles [bounds[x], bounds[x+1]), a
+// range of about an eighth of the estimated cost.  (Cutting the last tiles of a range into smaller pieces, so
 // that its CUs run dry together, was measured and does not pay: the pieces are
 // less efficient than what they save.)
 constexpr int kGemmTileNb = 8;  // column blocks (of 32) per tile of the grouped GEMMs
+constexpr int kRowTileGroup = 4;  // row tiles of one expert that run side by side (see write_expert_tiles)
 constexpr int kXcds = 8;
 // estimated cost of a tile: kCostPerTile + kCostPerRowBlock * row blocks.  The
 // fixed part (4 row blocks' worth) was fitted on measured runs with even,

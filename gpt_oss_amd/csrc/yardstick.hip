@@ -60,27 +60,40 @@ __global__ __launch_bounds__(256) void mfma_loop_kernel(int iters, int data, uns
   }
 }
 
-// dst[i] = src[i], 16 bytes per lane, grid-stride
+// dst = src: every wave takes blocks of 16 KB in turn, 16 loads of 1 KB in flight, then 16 stores
 __global__ __launch_bounds__(256) void copy_kernel(const uint4 *__restrict__ src, uint4 *__restrict__ dst,
                                                    size_t n) {
-  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256)
-    dst[i] = src[i];
+  const int lane = threadIdx.x & 63;
+  const size_t wave = (size_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  const size_t n_waves = (size_t)gridDim.x * 4;
+  const size_t n_blocks = n / 1024;  // 16 KB = 1024 uint4
+  for (size_t b = wave; b < n_blocks; b += n_waves) {
+    const uint4 *p = src + b * 1024 + lane;
+    uint4 *q = dst + b * 1024 + lane;
+    uint4 v[16];
+#pragma unroll
+    for (int j = 0; j < 16; j++) v[j] = p[j * 64];
+#pragma unroll
+    for (int j = 0; j < 16; j++) q[j * 64] = v[j];
+  }
 }
 
-// reads src once, 4 x 16 bytes per lane in flight, and keeps one word per workgroup
+// reads src once: every wave takes blocks of 16 KB in turn, 16 loads of 1 KB in
+// flight each, and keeps one word per workgroup
 __global__ __launch_bounds__(256) void read_kernel(const uint4 *__restrict__ src, uint32_t *__restrict__ sink,
                                                    size_t n) {
   uint32_t x = 0;
-  const size_t stride = (size_t)gridDim.x * 256;
-  size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
-  for (; i + 3 * stride < n; i += 4 * stride) {
-    const uint4 v0 = src[i], v1 = src[i + stride], v2 = src[i + 2 * stride], v3 = src[i + 3 * stride];
-    x ^= v0.x ^ v0.y ^ v0.z ^ v0.w ^ v1.x ^ v1.y ^ v1.z ^ v1.w ^ v2.x ^ v2.y ^ v2.z ^ v2.w ^ v3.x ^ v3.y ^
-         v3.z ^ v3.w;
-  }
-  for (; i < n; i += stride) {
-    const uint4 v = src[i];
-    x ^= v.x ^ v.y ^ v.z ^ v.w;
+  const int lane = threadIdx.x & 63;
+  const size_t wave = (size_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  const size_t n_waves = (size_t)gridDim.x * 4;
+  const size_t n_blocks = n / 1024;  // 16 KB = 1024 uint4
+  for (size_t b = wave; b < n_blocks; b += n_waves) {
+    const uint4 *p = src + b * 1024 + lane;
+    uint4 v[16];
+#pragma unroll
+    for (int j = 0; j < 16; j++) v[j] = p[j * 64];
+#pragma unroll
+    for (int j = 0; j < 16; j++) x ^= v[j].x ^ v[j].y ^ v[j].z ^ v[j].w;
   }
   if (x == 0x12345678u) sink[blockIdx.x] = x;
 }
@@ -144,14 +157,14 @@ done:
 }
 
 extern "C" int moe_yardstick_hbm(size_t bytes, int iters, double *copy_gbs, double *read_gbs) {
-  if (bytes < (1u << 20) || (bytes & 15) || iters < 1 || iters > 1000 || !copy_gbs || !read_gbs)
+  if (bytes < (1u << 20) || (bytes & 16383) || iters < 1 || iters > 1000 || !copy_gbs || !read_gbs)
     return set_error(MOE_ERR_BAD_ARG, "moe_yardstick_hbm: bad arguments");
   int rc = MOE_OK;
   uint4 *src = nullptr, *dst = nullptr;
   uint32_t *sink = nullptr;
   hipEvent_t e0 = nullptr, e1 = nullptr, e2 = nullptr;
   const size_t n = bytes / 16;
-  const int grid = 256 * 16;
+  const int grid = 256 * 8;
   float ms_copy = 0.f, ms_read = 0.f;
   Y_TRY(hipMalloc(reinterpret_cast<void **>(&src), bytes));
   Y_TRY(hipMalloc(reinterpret_cast<void **>(&dst), bytes));
