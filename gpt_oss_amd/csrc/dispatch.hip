@@ -1,5 +1,5 @@
-// Token -> expert dispatch: LDS histogram, prefix sum, stable permutation, and
-// the copy of the routed rows into per-expert segments.  Replaces
+// Token -> expert dispatch: LDS histogram, prefix sum, stable permutation and
+// the tile plan of the grouped GEMMs, and the combine that ends the layer.  Replaces
 // count_expert_assignments_kernel, exclusive_scan_small_kernel and
 // build_expert_assignments_kernel (utility/utility.cpp:1058-1106, :758-777),
 // whose order inside an expert segment is the order global atomics happen to
@@ -94,9 +94,13 @@ __device__ __forceinline__ void write_expert_tiles(int ee, int nmt, int rbe, int
   }
 }
 
+// write_global: this workgroup stores the plan (offsets, per-expert records,
+// totals, XCD bounds); the others only need the values returned to them.
+// with_tiles: this workgroup also writes the tile tables of all experts.
 __device__ __forceinline__ int build_plan(int count, int E, int n_ct_gate_up, int n_ct_down,
                                           const PlanOut &out, bool with_tiles, int *ex_count_out,
-                                          int *tot_count_out = nullptr) {
+                                          int *tot_count_out = nullptr, bool write_global = true,
+                                          ExpertInfo *info_out = nullptr) {
   __shared__ int sh_wave[4][4];  // [wave][quantity]: the waves' sums
   __shared__ int sh_nmt[256], sh_rb[256], sh_extra[256], sh_rowblk[256];
   __shared__ int sh_cost[257];   // exclusive prefix of the experts' cost per column tile
@@ -148,8 +152,7 @@ __device__ __forceinline__ int build_plan(int count, int E, int n_ct_gate_up, in
   }
   const int ex_count = ex[0], ex_pad = ex[1], ex_mt = ex[2], ex_cost = ex[3];
   const int tot_count = tot[0], tot_pad = tot[1], tot_mt = tot[2], tot_cost = tot[3];
-  if (e < E) {
-    offsets[e] = ex_count;
+  {
     ExpertInfo inf;
     inf.row0 = ex_pad;
     inf.rows = count;
@@ -158,7 +161,16 @@ __device__ __forceinline__ int build_plan(int count, int E, int n_ct_gate_up, in
     inf.tile_base = ex_mt;
     inf.extra = extra;
     inf.pad_[0] = inf.pad_[1] = 0;
-    info[e] = inf;
+    if (e < E && write_global) {
+      offsets[e] = ex_count;
+      info[e] = inf;
+    }
+    if (info_out) *info_out = inf;
+  }
+  if (!write_global) {  // (the same for the whole workgroup)
+    *ex_count_out = ex_count;
+    if (tot_count_out) *tot_count_out = tot_count;
+    return ex_pad;
   }
   sh_cost[e] = ex_cost;
   sh_tiles[e] = ex_mt;
@@ -207,7 +219,7 @@ __device__ __forceinline__ int build_plan(int count, int E, int n_ct_gate_up, in
     }
     sh_bound[g][x] = bound;
   }
-  // The tile sequences (three-launch form: written by the scatter kernel's
+  // The tile sequences (two-launch form: written by the scatter kernel's
   // workgroups instead, which are many).  The waves take the experts in turn.
   if (with_tiles) {
     for (int ee = w; ee < E; ee += 4)
@@ -237,37 +249,13 @@ __device__ __forceinline__ int build_plan(int count, int E, int n_ct_gate_up, in
   return ex_pad;
 }
 
-// Pass 2 (one workgroup): turns the per-workgroup counts into exclusive bases,
-// and builds per-expert offsets and the row-tile plan of the grouped GEMMs.
-// An expert with M rows has ceil(M / 32) row blocks, cut into n_mt = ceil(row
-// blocks / 8) tiles as evenly as they go: the first `extra` tiles are rb + 1
-// row blocks high, the others rb.  Its segment in the padded row space is its
-// row blocks and no more, so an expert pads to at most 31 rows.
-//
-// It also cuts the tile sequence of either GEMM (n_ct column tiles per row
-// tile) into the 8 ranges of the XCDs, by estimated cost: a tile of r row blocks
-// costs kCostPerTile + kCostPerRowBlock * r.
-__global__ __launch_bounds__(256) void dispatch_scan_kernel(int *__restrict__ blk_counts, int n_blk,
-                                                           int E, int n_ct_gate_up, int n_ct_down,
-                                                           PlanOut out) {
-  const int e = threadIdx.x;
-  int count = 0;
-  if (e < E) {
-    // 16 independent loads at a time, then their running sums back in place
-    for (int b0 = 0; b0 < n_blk; b0 += 16) {
-      int c[16];
-#pragma unroll
-      for (int i = 0; i < 16; i++) c[i] = b0 + i < n_blk ? blk_counts[(size_t)(b0 + i) * E + e] : 0;
-#pragma unroll
-      for (int i = 0; i < 16; i++) {
-        if (b0 + i < n_blk) blk_counts[(size_t)(b0 + i) * E + e] = count;
-        count += c[i];
-      }
-    }
-  }
-  int ex_count;
-  build_plan(count, E, n_ct_gate_up, n_ct_down, out, /*with_tiles=*/false, &ex_count);
-}
+// The row-tile plan (see build_plan): an expert with M rows has ceil(M / 32) row
+// blocks, cut into n_mt = ceil(row blocks / 8) tiles as evenly as they go: the
+// first `extra` tiles are rb + 1 row blocks high, the others rb.  Its segment in
+// the padded row space is its row blocks and no more, so an expert pads to at
+// most 31 rows.  The tile sequence of either GEMM (n_ct column tiles per row
+// tile) is cut into the 8 ranges of the XCDs by estimated cost: a tile of r row
+// blocks costs kCostPerTile + kCostPerRowBlock * r.
 
 // Ranks inside one wave: for each of the lane's kTopK expert ids, how many of
 // the wave's assignments to the same expert come before it in (lane, slot)
@@ -313,26 +301,27 @@ __device__ __forceinline__ void wave_ranks_for(int E, const int (&id)[kTopK], in
   else wave_ranks<8>(id, lane, rank, total);
 }
 
-// Pass 3: rank of every assignment inside its expert = (assignments of lower
-// workgroups) + (lower waves of this workgroup) + (lower lanes of this wave)
-// + (lower slots of this token), all for the same expert.
+// Pass 2: the plan and the stable permutation in one launch.  Every workgroup
+// adds up the per-workgroup counts of pass 1 itself (at most a few dozen loads
+// per expert): the experts' totals, from which it derives offsets and padded
+// first rows exactly as workgroup 0 does, and the counts of the workgroups
+// before it, its own base inside every expert.  Workgroup 0 also stores the
+// plan for the GEMMs; a one-workgroup kernel between the passes did that before
+// and cost a launch more than the repeated sums cost here.
+// Rank of an assignment inside its expert = (assignments of lower workgroups)
+// + (lower waves of this workgroup) + (lower lanes of this wave) + (lower slots
+// of this token), all for the same expert.
 __global__ __launch_bounds__(kDispThreads) void dispatch_scatter_kernel(
     const int *__restrict__ topk_i, const int *__restrict__ pos, int T, int E,
-    const int *__restrict__ blk_base, const int *__restrict__ offsets,
-    const ExpertInfo *__restrict__ info, int *__restrict__ perm, int *__restrict__ rowmap,
+    const int *__restrict__ blk_counts, int n_blk, int *__restrict__ perm, int *__restrict__ rowmap,
     int *__restrict__ inv, int n_ct_gate_up, int n_ct_down, PlanOut plan) {
   __shared__ int wave_cnt[kDispThreads / 64][256];
+  __shared__ int sh_base[256], sh_off[256], sh_row0[256];
+  __shared__ ExpertInfo sh_info[256];
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int w = tid >> 6;
-  // The tile sequences of the GEMMs, from the per-expert records of the scan
-  // kernel: the waves of all workgroups take the experts in turn (in the one
-  // workgroup of the scan kernel this took as long as everything else in it).
-  for (int ee = blockIdx.x * (kDispThreads / 64) + w; ee < E; ee += gridDim.x * (kDispThreads / 64)) {
-    const ExpertInfo inf = info[ee];
-    write_expert_tiles(ee, inf.n_mt, inf.rb, inf.extra, inf.row0 / kRowBlock, inf.tile_base, lane,
-                       n_ct_gate_up, n_ct_down, plan);
-  }
+  // the token's ids first: their loads run while the counts are added up
   const int t = blockIdx.x * kDispThreads + tid;
   int id[kTopK] = {-1, -1, -1, -1};
   if (t < T && !(pos && pos[t] < 0)) {
@@ -342,10 +331,38 @@ __global__ __launch_bounds__(kDispThreads) void dispatch_scatter_kernel(
     for (int k = 0; k < kTopK; k++)
       if (id[k] >= E) id[k] = -1;
   }
+  int count = 0, base = 0;
+  if (tid < E) {
+    for (int b0 = 0; b0 < n_blk; b0 += 16) {  // 16 independent loads at a time
+      int c[16];
+#pragma unroll
+      for (int i = 0; i < 16; i++) c[i] = b0 + i < n_blk ? blk_counts[(size_t)(b0 + i) * E + tid] : 0;
+#pragma unroll
+      for (int i = 0; i < 16; i++) {
+        if (b0 + i < (int)blockIdx.x) base += c[i];
+        count += c[i];
+      }
+    }
+  }
+  int ex_count;
+  ExpertInfo inf;
+  const int row0 = build_plan(count, E, n_ct_gate_up, n_ct_down, plan, /*with_tiles=*/false, &ex_count, nullptr,
+                              /*write_global=*/blockIdx.x == 0, &inf);
+  sh_base[tid] = base;
+  sh_off[tid] = ex_count;
+  sh_row0[tid] = row0;
+  sh_info[tid] = inf;
   for (int e = tid; e < (kDispThreads / 64) * 256; e += kDispThreads) (&wave_cnt[0][0])[e] = 0;
   int rank[kTopK], total[kTopK];
   wave_ranks_for(E, id, lane, rank, total);
   __syncthreads();
+  // The tile sequences of the GEMMs: the waves of all workgroups take the
+  // experts in turn.
+  for (int ee = blockIdx.x * (kDispThreads / 64) + w; ee < E; ee += gridDim.x * (kDispThreads / 64)) {
+    const ExpertInfo f = sh_info[ee];
+    write_expert_tiles(ee, f.n_mt, f.rb, f.extra, f.row0 / kRowBlock, f.tile_base, lane, n_ct_gate_up,
+                       n_ct_down, plan);
+  }
 #pragma unroll
   for (int k = 0; k < kTopK; k++)
     if (id[k] >= 0) wave_cnt[w][id[k]] = total[k];  // the same value from every lane that holds the id
@@ -357,10 +374,10 @@ __global__ __launch_bounds__(kDispThreads) void dispatch_scatter_kernel(
     const int e = id[k];
     const int a = t * kTopK + k;
     if (e < 0) { out_inv[k] = -1; continue; }
-    int r = blk_base[(size_t)blockIdx.x * E + e] + rank[k];
+    int r = sh_base[e] + rank[k];
     for (int ww = 0; ww < w; ww++) r += wave_cnt[ww][e];
-    const int prow = info[e].row0 + r;
-    perm[offsets[e] + r] = a;
+    const int prow = sh_row0[e] + r;
+    perm[sh_off[e] + r] = a;
     rowmap[prow] = a;
     out_inv[k] = prow;
   }
@@ -368,8 +385,8 @@ __global__ __launch_bounds__(kDispThreads) void dispatch_scatter_kernel(
       make_int4(out_inv[0], out_inv[1], out_inv[2], out_inv[3]);
 }
 
-// Passes 1-3 in one workgroup for batches of at most kSmallRounds x 256 tokens:
-// the rounds of 256 tokens play the part of the workgroups of the three-kernel
+// Both passes in one workgroup for batches of at most kSmallRounds x 256 tokens:
+// the rounds of 256 tokens play the part of the workgroups of the two-kernel
 // form (round r's assignments come after those of the rounds before it), so
 // the result is the same, bit for bit.
 constexpr int kSmallRounds = 1;
@@ -549,17 +566,15 @@ hipError_t launch_dispatch(const int *topk_i, const int *pos, int T, int E, int 
   plan.tile_cap_gate_up = d.tile_cap_gate_up;
   plan.tile_cap_down = d.tile_cap_down;
   if (n_blk <= kSmallRounds) {
-    // small batches: one workgroup does all three passes, two launches fewer
+    // small batches: one workgroup does both passes, one launch fewer
     dispatch_small_kernel<<<1, kDispThreads, 0, s>>>(topk_i, pos, T, E, n_ct_gate_up, n_ct_down, plan,
                                                      d.perm, d.rowmap, d.inv);
     return hipGetLastError();
   }
   dispatch_count_kernel<<<n_blk, kDispThreads, 0, s>>>(topk_i, pos, T, E, d.blk_counts, d.rowmap,
                                                        fill_rows, d.perm);
-  dispatch_scan_kernel<<<1, 256, 0, s>>>(d.blk_counts, n_blk, E, n_ct_gate_up, n_ct_down, plan);
-  dispatch_scatter_kernel<<<n_blk, kDispThreads, 0, s>>>(topk_i, pos, T, E, d.blk_counts, d.offsets,
-                                                         d.info, d.perm, d.rowmap, d.inv, n_ct_gate_up,
-                                                         n_ct_down, plan);
+  dispatch_scatter_kernel<<<n_blk, kDispThreads, 0, s>>>(topk_i, pos, T, E, d.blk_counts, n_blk, d.perm,
+                                                         d.rowmap, d.inv, n_ct_gate_up, n_ct_down, plan);
   return hipGetLastError();
 }
 

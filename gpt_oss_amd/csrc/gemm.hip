@@ -15,7 +15,7 @@
 // Tiling.  A workgroup of NW waves owns a tile of (RBT*32) rows x
 // (NW*NBW*32) columns of one expert.  The waves split the columns only: each
 // wave keeps RBT x NBW accumulators of 32x32 over all rows of the tile, RBT =
-// 1..8 following the expert's row count (see dispatch_scan_kernel), so a ragged
+// 1..8 following the expert's row count (see build_plan in dispatch.hip), so a ragged
 // segment pads to at most 31 rows and MFMA work follows the real rows.
 //
 // Feeding the matrix cores.  A step of 32 k needs 32 KB per CU, and one CU
@@ -928,7 +928,7 @@ __global__ __launch_bounds__(C::THREADS, C::WAVES) void grouped_gemm_kernel(
 // 256 accumulation registers); 256 x 256 tiles; 4 ring slots.
 using CfgGemm = GemmCfg<4, 2, 4>;
 static_assert(CfgGemm::RBT_MAX * kRowBlock == kTileRows && CfgGemm::TILE_NB == kGemmTileNb,
-              "tile plan of dispatch_scan_kernel");
+              "tile plan of build_plan");
 // Batches of at most 64 tokens: no expert has more than 64 rows, every tile is
 // one or two row blocks high and the GEMMs are a stream of weights.  What
 // limits that stream is the bytes one CU keeps in flight, so the same kernel is
