@@ -229,17 +229,20 @@ def main():
     # and on plain streams through HBM, measured now by the library's yardsticks.
     roofline["peak_kind"] = "published"
     try:
-        tf, ghz = abi.yardstick_mfma(256, 20000, data=True)
-        tf0, ghz0 = abi.yardstick_mfma(256, 20000, data=False)
+        tf, ghz = abi.yardstick_mfma(256, 20000, data=2)   # activations against weights, as in the layer
+        tf1, ghz1 = abi.yardstick_mfma(256, 20000, data=1)  # both operands of unit scale
+        tf0, ghz0 = abi.yardstick_mfma(256, 20000, data=0)
         copy_gbs, read_gbs = abi.yardstick_hbm(1 << 30, 10)
         roofline["measured_peak_tflops"] = tf
         roofline["measured_peak_gbs"] = max(copy_gbs, read_gbs)
         roofline["measured_peak"] = {
             "mfma_tflops": tf, "mfma_shader_ghz": ghz,
+            "mfma_tflops_unit_scale_operands": tf1, "mfma_shader_ghz_unit_scale_operands": ghz1,
             "mfma_tflops_zero_operands": tf0, "mfma_shader_ghz_zero_operands": ghz0,
             "hbm_copy_gbs": copy_gbs, "hbm_read_gbs": read_gbs,
             "how": "moe_yardstick_mfma: v_mfma_f32_32x32x16_bf16 from registers, 256 workgroups x 4 waves, "
-                   "16 accumulators each; moe_yardstick_hbm: copy (read + write bytes) and read-only "
+                   "16 accumulators each, pseudo-random operands (unit scale against scale 0.02, as "
+                   "activations meet weights); moe_yardstick_hbm: copy (read + write bytes) and read-only "
                    "kernels over 1 GiB"}
         roofline["frac_of_measured_peak"] = (mfma_tflops / tf if roofline["bound"] == "mfma"
                                              else hbm_gbs / max(copy_gbs, read_gbs))

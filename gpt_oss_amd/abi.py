@@ -147,10 +147,11 @@ def dispatch_static(topk_i, pos, n_tokens, n_experts, offsets, perm, stream=None
                                     stream))
 
 
-def yardstick_mfma(n_workgroups: int = 256, iters: int = 20000, data: bool = True):
-    """(TFLOP/s, shader GHz) of a register-resident v_mfma_f32_32x32x16_bf16 loop."""
+def yardstick_mfma(n_workgroups: int = 256, iters: int = 20000, data: int = 1):
+    """(TFLOP/s, shader GHz) of a register-resident v_mfma_f32_32x32x16_bf16 loop.
+    data: 0 zeros, 1 operands of unit scale, 2 unit scale against scale 0.02."""
     tf, ghz = C.c_double(), C.c_double()
-    check(lib().moe_yardstick_mfma(n_workgroups, iters, 1 if data else 0, C.byref(tf), C.byref(ghz)))
+    check(lib().moe_yardstick_mfma(n_workgroups, iters, int(data), C.byref(tf), C.byref(ghz)))
     return float(tf.value), float(ghz.value)
 
 

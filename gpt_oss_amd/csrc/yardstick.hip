@@ -19,9 +19,10 @@ typedef float yf32x16 __attribute__((ext_vector_type(16)));
 
 // 4 waves per workgroup, one per SIMD, each with 16 independent accumulators of
 // v_mfma_f32_32x32x16_bf16 (all 256 accumulation registers, as a GEMM tile) and
-// no memory traffic at all.  The operands are pseudo-random values of unit
-// scale (data != 0) or zeros: the clock the matrix cores sustain depends on how
-// many bits toggle.  out[2*wg] = shader clocks, out[2*wg+1] = ticks of the
+// no memory traffic at all.  The operands are pseudo-random values (data 1: unit
+// scale; data 2: unit scale against a scale of 0.02, as activations meet
+// weights in the layer) or zeros (data 0): the clock the matrix cores sustain
+// depends on how many bits toggle.  out[2*wg] = shader clocks, out[2*wg+1] = ticks of the
 // constant 100 MHz clock spent in the loop by the workgroup's first wave.
 __global__ __launch_bounds__(256) void mfma_loop_kernel(int iters, int data, unsigned long long *out,
                                                         float *sink) {
@@ -36,12 +37,18 @@ __global__ __launch_bounds__(256) void mfma_loop_kernel(int iters, int data, uns
   for (int h = 0; h < 2; h++)
 #pragma unroll
     for (int j = 0; j < 8; j++) {
-      s = s * 1664525u + 1013904223u;
-      const float u = (float)(s >> 8) * (1.0f / 8388608.0f) - 1.0f;  // [-1, 1)
-      s = s * 1664525u + 1013904223u;
-      const float v = (float)(s >> 8) * (1.0f / 8388608.0f) - 1.0f;
-      a[h][j] = (__bf16)(data ? 1.7f * u : 0.f);
-      b[h][j] = (__bf16)(data ? 1.7f * v : 0.f);
+      float u = 0.f, v = 0.f;  // sums of four uniform variates on [-1, 1): bell-shaped, variance 4/3
+#pragma unroll
+      for (int r = 0; r < 4; r++) {
+        s = s * 1664525u + 1013904223u;
+        u += (float)(s >> 8) * (1.0f / 8388608.0f) - 1.0f;
+        s = s * 1664525u + 1013904223u;
+        v += (float)(s >> 8) * (1.0f / 8388608.0f) - 1.0f;
+      }
+      // data 1: both operands of unit scale; data 2: as the layer's GEMMs see them,
+      // activations of unit scale against weights of scale 0.02; data 0: zeros
+      a[h][j] = (__bf16)(data ? 0.866f * u : 0.f);
+      b[h][j] = (__bf16)(data == 1 ? 0.866f * v : (data == 2 ? 0.0173f * v : 0.f));
     }
   const unsigned long long c0 = clock64(), t0 = wall_clock64();
   for (int it = 0; it < iters; it++) {

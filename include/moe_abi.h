@@ -279,9 +279,10 @@ int moe_time_forward_each(moe_handle *h, int layer, const uint16_t *x,
  * moe_yardstick_mfma: n_workgroups workgroups of 4 waves (one per SIMD, one
  * workgroup per CU up to the CU count) run v_mfma_f32_32x32x16_bf16 on 16
  * independent accumulators each from registers alone, iters x 16 per wave.
- * data != 0: pseudo-random operands of unit scale; data == 0: zeros (the clock
- * the matrix cores sustain depends on the bits that toggle).  Returns TFLOP/s
- * over the launch and the mean shader clock in GHz during the loop.
+ * data 1: pseudo-random operands of unit scale; data 2: unit scale against a
+ * scale of 0.02, as activations meet weights in the layer; data 0: zeros (the
+ * clock the matrix cores sustain depends on the bits that toggle).  Returns
+ * TFLOP/s over the launch and the mean shader clock in GHz during the loop.
  *
  * moe_yardstick_hbm: a copy kernel and a read-only kernel over `bytes` of
  * device memory (choose it well above the 256 MB memory-side cache), iters

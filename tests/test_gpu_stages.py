@@ -170,9 +170,10 @@ def test_yardsticks_run():
     """The measured denominators the benchmark reports: a register-resident MFMA
     loop and plain streams through HBM.  Sanity only: positive, below the
     published peaks, zeros no slower than random operands."""
-    tf, ghz = abi.yardstick_mfma(256, 2000, data=True)
-    tf0, _ = abi.yardstick_mfma(256, 2000, data=False)
-    assert 200 < tf < 2600 and 0.5 < ghz < 3.0 and tf0 > 0.9 * tf
+    tf, ghz = abi.yardstick_mfma(256, 2000, data=1)
+    tf2, _ = abi.yardstick_mfma(256, 2000, data=2)
+    tf0, _ = abi.yardstick_mfma(256, 2000, data=0)
+    assert 200 < tf < 2600 and 200 < tf2 < 2600 and 0.5 < ghz < 3.0 and tf0 > 0.9 * tf
     c, r = abi.yardstick_hbm(1 << 28, 3)
     assert 500 < c < 8200 and 500 < r < 8200
 
