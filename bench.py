@@ -10,8 +10,9 @@ the timed steps, and the CPU baseline (the reference's CPU/OpenMP path) timed on
 this host on a bounded prefix of the same batch.  At the default workload the
 line also carries "decode_mxfp4", a side figure for the decode-regime
 configuration (64 tokens, MXFP4 expert weights; `--workload c5` makes that
-configuration the one measured), and "prefill_mxfp4", the headline batch with
-MXFP4 expert weights.  Neither is part of `value`.
+configuration the one measured), "prefill_mxfp4", the headline batch with
+MXFP4 expert weights, and "other_workloads", short legs of the remaining
+benchmark configurations (c3a, c3b, c4).  None of them is part of `value`.
 """
 from __future__ import annotations
 
@@ -172,6 +173,36 @@ def run_leg(shape, steps, warmup, device_timed=False, mxfp4=None):
     return elapsed / steps, stages, n_meas, float(np.median(each)) * 1e-3, L
 
 
+def side_leg(name, steps=60, warmup=10):
+    """One of the other benchmark configurations as a side figure of the default
+    line: tokens/s, stage times and the gate_up GEMM against the roofline that
+    binds it (published peaks), measured like the headline workload."""
+    shape = synth_configs()[name]
+    T, H, IM, E, K = shape.tokens, shape.hidden, shape.inter, shape.experts, shape.topk
+    s_step, st, _, med, _ = run_leg(shape, steps, warmup)
+    A = T * K
+    t_gu, t_dn = st["gate_up"] * 1e-3, st["down"] * 1e-3
+    fl_gu, fl_dn = 2.0 * A * H * 2 * IM, 2.0 * A * IM * H
+    by_gu = E * 2 * IM * H * 2.0 + A * H * 2 + A * IM * 2
+    by_dn = E * H * IM * 2.0 + A * IM * 2 + A * H * 4
+    bound = BOUND[name]
+    ach = fl_gu / t_gu / 1e12 if bound == "mfma" else by_gu / t_gu / 1e9
+    return {"workload": f"{name}: {T} tokens, {E} experts, bf16 weights" + (", Zipf(1.2) routing" if shape.zipf else ""),
+            "tokens_per_s": T / s_step, "us_per_step": s_step * 1e6, "median_us_per_step": med * 1e6,
+            "stage_us": {k: v * 1e3 for k, v in st.items()},
+            "gate_up_roofline": {"bound": bound, "achieved": ach, "unit": "TFLOP/s" if bound == "mfma" else "GB/s",
+                                 "frac": ach / (PEAK_BF16_TFLOPS if bound == "mfma" else PEAK_HBM_GBS)},
+            "expert_gemms": {"tflops": (fl_gu + fl_dn) / (t_gu + t_dn) / 1e12,
+                             "frac_bf16_peak": (fl_gu + fl_dn) / (t_gu + t_dn) / 1e12 / PEAK_BF16_TFLOPS,
+                             "gbs": (by_gu + by_dn) / (t_gu + t_dn) / 1e9,
+                             "frac_hbm_peak": (by_gu + by_dn) / (t_gu + t_dn) / 1e9 / PEAK_HBM_GBS}}
+
+
+def synth_configs():
+    from gpt_oss_amd import synth
+    return synth.CONFIGS
+
+
 def mxfp4_weight_bytes(shape):
     # nibbles + one scale byte per 32 weights
     return shape.experts * 3 * shape.hidden * shape.inter * (0.5 + 1.0 / 32)
@@ -185,7 +216,8 @@ def main():
     ap.add_argument("--workload", default="c2", help="c2 (headline), c3a, c3b, c4, c5 (MXFP4 decode)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-decode", action="store_true",
-                    help="c2 only: skip the two side figures with MXFP4 weights (workload c5, and c2's batch)")
+                    help="c2 only: skip the side figures (MXFP4 weights: workload c5 and c2's batch; "
+                         "the other configurations c3a, c3b, c4)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)",
@@ -312,6 +344,9 @@ def main():
             "gate_up_frac_bf16_peak": flops_gate_up / tg / 1e12 / PEAK_BF16_TFLOPS,
             "expert_gemms_tflops": (flops_gate_up + flops_down) / (tg + td) / 1e12,
             "expert_gemms_frac_bf16_peak": (flops_gate_up + flops_down) / (tg + td) / 1e12 / PEAK_BF16_TFLOPS}
+        # The other benchmark configurations (skewed routing at 512 and 7168
+        # tokens, the 128-expert shape), each a short leg of its own.
+        result["other_workloads"] = {n: side_leg(n) for n in ("c3a", "c3b", "c4")}
     if not args.no_cpu_baseline and L is not None:
         result["cpu_baseline"] = cpu_baseline(shape, L)
     print(json.dumps(result))
