@@ -812,8 +812,8 @@ __device__ __forceinline__ void gemm_tile_gl(const uint4 *__restrict__ x_rows,  
   gate_up_epilogue<RBT, RS, C>(acc, outp, out_ld, limit, rb0, rbt, nb0, nb_valid, cw, rg, lane);
 }
 
-// DIRECT (small-batch configuration only): there is no plan.  Workgroup b is
-// column tile b % n_ct of expert b / n_ct; its 256 threads look at one
+// DIRECT (small-batch configuration only): there is no plan.  A workgroup is
+// one column tile of one expert (see the mapping below); its 256 threads look at one
 // assignment of the batch each and find the expert's rows with a ballot (see
 // DirectIds).  An expert without rows ends its workgroups here.
 template <typename C, bool GATE_UP, bool FP4, bool GATHER, bool DIRECT = false>
@@ -841,7 +841,13 @@ __global__ __launch_bounds__(C::THREADS, C::WAVES) void grouped_gemm_kernel(
   const int *map = rowmap;
   if constexpr (DIRECT) {
     const int tid = threadIdx.x;
-    const int e = blockIdx.x / n_ct;
+    // Workgroup ids are dealt round-robin to the 8 XCDs: XCD x takes the experts
+    // x, x + 8, ..., all column tiles of an expert, so that the expert's rows
+    // (which every one of its column tiles reads) are fetched into one L2
+    // instead of eight.
+    const int xcd = blockIdx.x & (kXcds - 1), idx = blockIdx.x >> 3;
+    const int e = (idx / n_ct) * kXcds + xcd;
+    if (e >= ids.E) return;  // surplus workgroups of the grid (experts not a multiple of 8)
     const bool mine = direct_expert_of(ids, tid) == e;
     const unsigned long long bal = __ballot(mine);
     if ((tid & 63) == 0) direct_cnt[tid >> 6] = __popcll(bal);
@@ -862,7 +868,7 @@ __global__ __launch_bounds__(C::THREADS, C::WAVES) void grouped_gemm_kernel(
       map = direct_rows;
     }
     tc.e = e;
-    tc.nt = blockIdx.x % n_ct;
+    tc.nt = idx % n_ct;
     tc.rb0 = e * (kDirectSlotRows / kRowBlock);
     tc.rbt = (min(count, kDirectSlotRows) + kRowBlock - 1) / kRowBlock;
   } else {
@@ -945,7 +951,7 @@ static hipError_t launch_gemm(const uint4 *a, const uint4 *w, const uint16_t *w_
                               float limit, int mt_cap, const DirectIds &direct, hipStream_t s) {
   const int nb_total = (GATE_UP ? 2 * N : N) / kRowBlock;
   const int n_ct = (nb_total + C::TILE_NB - 1) / C::TILE_NB;
-  const int grid = DIRECT ? direct.E * n_ct : kXcds * xcd_tile_cap(mt_cap * n_ct);
+  const int grid = DIRECT ? kXcds * ((direct.E + kXcds - 1) / kXcds) * n_ct : kXcds * xcd_tile_cap(mt_cap * n_ct);
   const TileDesc *tiles = GATE_UP ? d.tiles_gate_up : d.tiles_down;
   if (w_scale) {
     grouped_gemm_kernel<C, GATE_UP, true, GATHER, DIRECT><<<grid, C::THREADS, 0, s>>>(
