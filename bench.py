@@ -33,7 +33,7 @@ PEAK_HBM_GBS = 8000.0
 SETTLE_STEPS = 200  # untimed calls in front of the warm-up steps, see run_leg
 # which roofline binds the gate_up GEMM of a workload: rows per expert
 # (4 T / E) against the machine balance of 312 flop per byte
-BOUND = {"c2": "mfma", "c3a": "hbm", "c3b": "mfma", "c4": "hbm", "c5": "hbm"}
+BOUND = {"c2": "mfma", "c3a": "hbm", "c3b": "mfma", "c4": "hbm", "c5": "hbm", "d4": "mfma"}
 
 
 def cpu_model() -> str:
@@ -213,7 +213,8 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=500)
     ap.add_argument("--warmup", type=int, default=50)
-    ap.add_argument("--workload", default="c2", help="c2 (headline), c3a, c3b, c4, c5 (MXFP4 decode)")
+    ap.add_argument("--workload", default="c2",
+                    help="c2 (headline), c3a, c3b, c4, c5 (MXFP4 decode); d4: yardstick, four dense GEMMs of 4096 rows")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-decode", action="store_true",
                     help="c2 only: skip the side figures (MXFP4 weights: workload c5 and c2's batch; "

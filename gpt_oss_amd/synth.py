@@ -44,6 +44,10 @@ CONFIGS = {
     "c4": LayerShape("c4", 6144, 2880, 2880, 128),
     # 20B shape, expert matrices given as MXFP4 blocks and scales (make_experts_mxfp4)
     "c5": LayerShape("c5", 64, 2880, 2880, 32),
+    # Not a benchmark configuration: a yardstick.  Four experts and top-4, so every
+    # token goes to every expert and the grouped GEMMs are four dense ones of
+    # 4096 rows each: what the kernels reach without ragged segments.
+    "d4": LayerShape("d4", 4096, 2880, 2880, 4),
 }
 
 
