@@ -91,3 +91,18 @@ def test_synth_is_deterministic_and_thread_count_independent():
     assert abs(float(a.std()) - 0.02) < 2e-4
     x = synth.make_activations(synth.CONFIGS["c2"], tokens=8)
     np.testing.assert_allclose(np.sqrt((x.astype(np.float64) ** 2).mean(axis=1)), 1.0, atol=3e-3)
+
+
+def test_bench_refuses_more_than_one_gpu_and_needs_a_gpu():
+    """bench.py measures one GPU: --gpus 2 exits with a message saying so; with
+    no GPU visible it exits rather than falling back to anything."""
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"],
+                       capture_output=True, text=True, timeout=120)
+    assert r.returncode == 2 and "one GPU" in r.stderr
+    if abi.device_count() == 0:
+        r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--steps", "1", "--warmup", "0"],
+                           capture_output=True, text=True, timeout=120)
+        assert r.returncode == 3 and "no CPU fallback" in r.stderr and r.stdout.strip() == ""
