@@ -488,12 +488,16 @@ __global__ __launch_bounds__(kDispThreads) void dispatch_small_kernel(
 // DIRECT: there was no dispatch pass (see DirectIds).  The row of assignment
 // (t, k) is its expert's slot plus the number of lower assignments of the batch
 // with the same expert, which the workgroup's 256 threads count with a ballot.
-template <bool RESID, bool DIRECT>
+// SPLIT: the down GEMM summed its reduction in two parts (down_k_split); the
+// second part's rows lie part_stride floats behind the first's and are added to
+// them before the weighting.
+template <bool RESID, bool DIRECT, bool SPLIT>
 __global__ __launch_bounds__(256) void combine_kernel(const float *__restrict__ y,
                                                      const int *__restrict__ inv,
                                                      const float *__restrict__ topk_v,
                                                      const int *__restrict__ pos, void *outp, int H,
-                                                     int ldy, int accumulate, DirectIds ids) {
+                                                     int ldy, int accumulate, DirectIds ids,
+                                                     size_t part_stride) {
   const int t = blockIdx.x;
   const bool active = !(pos && pos[t] < 0);
   if (!active && (accumulate || RESID)) return;
@@ -533,7 +537,11 @@ __global__ __launch_bounds__(256) void combine_kernel(const float *__restrict__ 
 #pragma unroll
     for (int k = 0; k < kTopK; k++) {
       if (p[k] >= 0) {
-        const float4 v = reinterpret_cast<const float4 *>(y + (size_t)p[k] * ldy)[c];
+        float4 v = reinterpret_cast<const float4 *>(y + (size_t)p[k] * ldy)[c];
+        if (SPLIT) {
+          const float4 v2 = reinterpret_cast<const float4 *>(y + part_stride + (size_t)p[k] * ldy)[c];
+          v.x += v2.x; v.y += v2.y; v.z += v2.z; v.w += v2.w;
+        }
         s.x += w[k] * v.x; s.y += w[k] * v.y; s.z += w[k] * v.z; s.w += w[k] * v.w;
       }
     }
@@ -578,26 +586,36 @@ hipError_t launch_dispatch(const int *topk_i, const int *pos, int T, int E, int 
   return hipGetLastError();
 }
 
-hipError_t launch_combine(const float *y, int ldy, const int *inv, const float *topk_v, const int *pos,
-                          float *out, int T, int H, int accumulate, const DirectIds &direct,
-                          hipStream_t s) {
+template <bool RESID>
+static hipError_t launch_combine_any(const float *y, int ldy, int y_parts, size_t part_stride, const int *inv,
+                                     const float *topk_v, const int *pos, void *out, int T, int H,
+                                     int accumulate, const DirectIds &direct, hipStream_t s) {
+  static_assert(kSmallBatchKSplit == 2, "the combine adds two parts");
+  if (y_parts != 1 && y_parts != kSmallBatchKSplit) return hipErrorInvalidValue;
+  const bool split = y_parts == 2;
+#define MOE_COMBINE(DIRECT, SPLIT)                                                                             \
+  combine_kernel<RESID, DIRECT, SPLIT><<<T, 256, 0, s>>>(y, inv, topk_v, pos, out, H, ldy, accumulate, direct, \
+                                                         part_stride)
   if (direct.topk_i) {
-    combine_kernel<false, true><<<T, 256, 0, s>>>(y, inv, topk_v, pos, out, H, ldy, accumulate, direct);
+    if (split) MOE_COMBINE(true, true); else MOE_COMBINE(true, false);
   } else {
-    combine_kernel<false, false><<<T, 256, 0, s>>>(y, inv, topk_v, pos, out, H, ldy, accumulate, direct);
+    if (split) MOE_COMBINE(false, true); else MOE_COMBINE(false, false);
   }
+#undef MOE_COMBINE
   return hipGetLastError();
 }
 
-hipError_t launch_combine_residual(const float *y, int ldy, const int *inv, const float *topk_v,
-                                   const int *pos, uint16_t *x, int T, int H, const DirectIds &direct,
-                                   hipStream_t s) {
-  if (direct.topk_i) {
-    combine_kernel<true, true><<<T, 256, 0, s>>>(y, inv, topk_v, pos, x, H, ldy, 0, direct);
-  } else {
-    combine_kernel<true, false><<<T, 256, 0, s>>>(y, inv, topk_v, pos, x, H, ldy, 0, direct);
-  }
-  return hipGetLastError();
+hipError_t launch_combine(const float *y, int ldy, int y_parts, size_t part_stride, const int *inv,
+                          const float *topk_v, const int *pos, float *out, int T, int H, int accumulate,
+                          const DirectIds &direct, hipStream_t s) {
+  return launch_combine_any<false>(y, ldy, y_parts, part_stride, inv, topk_v, pos, out, T, H, accumulate, direct,
+                                   s);
+}
+
+hipError_t launch_combine_residual(const float *y, int ldy, int y_parts, size_t part_stride, const int *inv,
+                                   const float *topk_v, const int *pos, uint16_t *x, int T, int H,
+                                   const DirectIds &direct, hipStream_t s) {
+  return launch_combine_any<true>(y, ldy, y_parts, part_stride, inv, topk_v, pos, x, T, H, 0, direct, s);
 }
 
 }  // namespace moe

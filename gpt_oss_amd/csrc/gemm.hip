@@ -229,6 +229,9 @@ __device__ __forceinline__ void gemm_tile(const uint4 *__restrict__ a_frag,  // 
                                           const uint4 *__restrict__ b_frag,  // expert: [nb][KB][64], FP4: [nb/2][KB/2][64]
                                           const uint16_t *__restrict__ b_scale,  // FP4: expert's [nb/2][KB/2][32] byte pairs
                                           int KB, int rb0, int rbt, int nb0, int nb_valid,
+                                          // the part of the reduction this workgroup sums: steps (of 32 k)
+                                          // [ks_begin, ks_begin + ks_count); the bias goes in with the first
+                                          int ks_begin, int ks_count,
                                           const int *__restrict__ rowmap,    // GATHER: padded row -> assignment
                                           int map_rb0,                       // row block that rowmap[0] belongs to
                                           const float *__restrict__ bias_a,  // gate / down bias (expert)
@@ -300,12 +303,13 @@ __device__ __forceinline__ void gemm_tile(const uint4 *__restrict__ a_frag,  // 
   } else {
 #pragma unroll
     for (int j = 0; j < NBW; j++)
-      bias_d[j] = bias_a[kRowBlock * (nb0 + min(cw * NBW + j, nb_valid - 1)) + (lane & 31)];
+      bias_d[j] = ks_begin == 0 ? bias_a[kRowBlock * (nb0 + min(cw * NBW + j, nb_valid - 1)) + (lane & 31)] : 0.f;
   }
   f32x16 acc[RBT][NBW];
 
-  const int n_steps = KB / KPS;
-  const uint4 *a_src = a_frag + (size_t)rb0 * KB * 64 + lane;
+  const int steps_total = KB / KPS;
+  const int n_steps = ks_count;
+  const uint4 *a_src = a_frag + ((size_t)rb0 * KB + ks_begin * KPS) * 64 + lane;
   // GATHER: per DMA of a step, this lane's place in its token's row (16-byte
   // units: a row is KB * 2 of them, a k block 2, the lane's half of it 1).
   // Padding rows read token 0; their products are never used.
@@ -317,7 +321,7 @@ __device__ __forceinline__ void gemm_tile(const uint4 *__restrict__ a_frag,  // 
       const int blk = RS == 1 ? c / KPS : min(c / KPS, rbt - 1);
       const int a = rowmap[(rb0 - map_rb0 + blk) * kRowBlock + (lane & 31)];
       const int tok = a >= 0 ? a / kTopK : 0;
-      lane_off[m] = (uint32_t)tok * (uint32_t)(KB * 2) + (c % KPS) * 2 + (lane >> 5);
+      lane_off[m] = (uint32_t)tok * (uint32_t)(KB * 2) + (ks_begin * KPS + c % KPS) * 2 + (lane >> 5);
     }
   }
   // Column blocks past the end of the matrix (last column tile only) re-load
@@ -326,12 +330,12 @@ __device__ __forceinline__ void gemm_tile(const uint4 *__restrict__ a_frag,  // 
   const uint16_t *s_src = nullptr;
   if (FP4) {
     const size_t pair = (size_t)((nb0 + min(cw * NBW, nb_valid - NBW)) >> 1);
-    b_src[0] = b_frag + pair * n_steps * 64 + lane;
-    s_src = b_scale + pair * n_steps * 32 + (lane & 31);
+    b_src[0] = b_frag + (pair * steps_total + ks_begin) * 64 + lane;
+    s_src = b_scale + (pair * steps_total + ks_begin) * 32 + (lane & 31);
   } else {
 #pragma unroll
     for (int j = 0; j < NBW; j++)
-      b_src[j] = b_frag + (size_t)(nb0 + min(cw * NBW + j, nb_valid - 1)) * KB * 64 + lane;
+      b_src[j] = b_frag + ((size_t)(nb0 + min(cw * NBW + j, nb_valid - 1)) * KB + ks_begin * KPS) * 64 + lane;
   }
 
   // Row operand: chunk c of a step (c = pass*NW + wave) is row block c / KPS, k block c % KPS.
@@ -510,6 +514,27 @@ __device__ __forceinline__ void gemm_tile(const uint4 *__restrict__ a_frag,  // 
   if (cw * NBW >= nb_valid) return;  // a wave without columns (last column tile only)
   if (GATE_UP) {
     gate_up_epilogue<RBT, RS, C>(acc, outp, out_ld, limit, rb0, rbt, nb0, nb_valid, cw, rg, lane);
+  } else if constexpr (C::RBT_MAX == 2) {
+    // Small-batch configuration: the rows go out straight from the accumulators
+    // (register q of lane l is token 8*(q/4) + 4*(l/32) + q%4, column l % 32: a
+    // store writes two rows of 128 contiguous bytes).  No LDS buffer, so that a
+    // third workgroup fits a CU; at full tile height the two forms take the same
+    // time.
+    static_assert(RS == 1, "the small-batch configuration has no row split");
+    float *y = reinterpret_cast<float *>(outp);
+    const int n = lane & 31;
+    const int rsub = 4 * (lane >> 5);
+#pragma unroll
+    for (int i = 0; i < RBT; i++) {
+      const size_t row0 = (size_t)(rb0 + i) * kRowBlock;
+#pragma unroll
+      for (int j = 0; j < NBW; j++) {
+        if (cw * NBW + j >= nb_valid) continue;
+        float *dst = y + row0 * out_ld + kRowBlock * (nb0 + cw * NBW + j) + n;
+#pragma unroll
+        for (int q = 0; q < 16; q++) dst[(size_t)(8 * (q >> 2) + rsub + (q & 3)) * out_ld] = acc[i][j][q];
+      }
+    }
   } else {
     constexpr int LD = C::EPI_LD;  // +8 floats keep the two lane halves on different banks
     float *y = reinterpret_cast<float *>(outp);
@@ -823,7 +848,7 @@ __global__ __launch_bounds__(C::THREADS, C::WAVES) void grouped_gemm_kernel(
     const float *__restrict__ bias_a, const float *__restrict__ bias_b,
     const TileDesc *__restrict__ tiles, const int *__restrict__ totals,
     const int *__restrict__ rowmap, void *__restrict__ outp, int K, int N, float limit,
-    DirectIds ids) {
+    DirectIds ids, size_t split_stride) {
   static_assert(!GATHER || GATE_UP, "only the first GEMM reads token rows");
   static_assert(!DIRECT || (C::RBT_MAX * kRowBlock == kDirectSlotRows && C::THREADS == kDirectTokens * kTopK),
                 "a direct batch: one thread per assignment, an expert's slot is one tile high");
@@ -831,7 +856,7 @@ __global__ __launch_bounds__(C::THREADS, C::WAVES) void grouped_gemm_kernel(
   static_assert(R <= 7, "seven stage arrays are declared below");
   __shared__ uint4 st0[C::STAGE], st1[C::STAGE], st2[C::STAGE], st3[C::STAGE], st4[C::STAGE],
       st5[C::STAGE], st6[C::STAGE], st7[C::STAGE];  // those a variant does not use take no room
-  __shared__ uint4 epi[C::NW * C::EPI_WAVE];
+  __shared__ uint4 epi[C::RBT_MAX == 2 ? 1 : C::NW * C::EPI_WAVE];  // the small-batch configuration stores directly
   const int KB = K / kFragK;
   const int nb_total = (GATE_UP ? 2 * N : N) / kRowBlock;  // weight row blocks per expert
   const int n_ct = (nb_total + C::TILE_NB - 1) / C::TILE_NB;
@@ -875,6 +900,14 @@ __global__ __launch_bounds__(C::THREADS, C::WAVES) void grouped_gemm_kernel(
     if (!locate_tile(tiles, totals + (GATE_UP ? kTotBoundsGateUp : kTotBoundsDown), tc)) return;
   }
   const int map_rb0 = DIRECT ? tc.rb0 : 0;
+  // The down GEMM of the small-batch configuration splits the reduction over
+  // gridDim.y workgroups; part p writes its sums to its own copy of the output,
+  // split_stride bytes behind the one before (the combine adds the parts up).
+  const int steps_total = K / (kFragK * C::KPS);
+  const int ks_per = (steps_total + (int)gridDim.y - 1) / (int)gridDim.y;
+  const int ks_begin = GATE_UP ? 0 : (int)blockIdx.y * ks_per;
+  const int ks_count = GATE_UP ? steps_total : min(ks_per, steps_total - ks_begin);
+  if (!GATE_UP) outp = static_cast<char *>(outp) + (size_t)blockIdx.y * split_stride;
   const int nb0 = tc.nt * C::TILE_NB;
   const int nb_valid = min(C::TILE_NB, nb_total - nb0);
   // per expert: bf16 nb_total * KB fragments of 1 KB; MXFP4 (nb_total/2) * (KB/2) chunks of 1 KB
@@ -891,8 +924,8 @@ __global__ __launch_bounds__(C::THREADS, C::WAVES) void grouped_gemm_kernel(
                                   outp, N, limit, st0, st1, st2, st3, st4, st5, st6, st7);                    \
     } else {                                                                                                  \
       gemm_tile<n, rs, C, GATE_UP, FP4, GATHER>(a_frag, b_frag, b_scale, KB, tc.rb0, tc.rbt, nb0, nb_valid,   \
-                                                map, map_rb0, ba, bb, outp, N, limit, st0, st1, st2, st3,     \
-                                                st4, st5, st6, epi);                                          \
+                                                ks_begin, ks_count, map, map_rb0, ba, bb, outp, N, limit,     \
+                                                st0, st1, st2, st3, st4, st5, st6, epi);                      \
     }                                                                                                         \
   } while (0)
 #define MOE_TILE(n) MOE_TILE_RS(n, 1)
@@ -941,24 +974,31 @@ static_assert(CfgGemm::RBT_MAX * kRowBlock == kTileRows && CfgGemm::TILE_NB == k
 // built with LDS stages for two row blocks and registers for two waves per
 // SIMD, and several workgroups share a CU.
 using CfgGemmSmall = GemmCfg<4, 2, 7, 2, 2>;
+using CfgGemmSmallFp4 = GemmCfg<4, 2, 7, 2, 3>;
 constexpr int kSmallBatchTokens = CfgGemmSmall::RBT_MAX * kRowBlock;
 
 // w_scale == nullptr: w holds bf16 fragments; otherwise w holds MXFP4 chunks and
 // w_scale their scale bytes (pack_fp4_kernel).
-template <typename C, bool GATE_UP, bool GATHER = false, bool DIRECT = false>
+// CF: the configuration of the MXFP4 instance (its column operand's ring takes a
+// third of the registers, so the small-batch down GEMM, which has no LDS buffer
+// for its output, can be held to three waves per SIMD; holding gate_up to the
+// same bound changes nothing in its register count and cost it 3 us per call).
+template <typename C, bool GATE_UP, bool GATHER = false, bool DIRECT = false, typename CF = C>
 static hipError_t launch_gemm(const uint4 *a, const uint4 *w, const uint16_t *w_scale, const float *ba,
                               const float *bb, const DispatchBuffers &d, void *out, int K, int N,
-                              float limit, int mt_cap, const DirectIds &direct, hipStream_t s) {
+                              float limit, int mt_cap, const DirectIds &direct, int k_split,
+                              size_t split_stride, hipStream_t s) {
   const int nb_total = (GATE_UP ? 2 * N : N) / kRowBlock;
   const int n_ct = (nb_total + C::TILE_NB - 1) / C::TILE_NB;
-  const int grid = DIRECT ? kXcds * ((direct.E + kXcds - 1) / kXcds) * n_ct : kXcds * xcd_tile_cap(mt_cap * n_ct);
+  const dim3 grid(DIRECT ? kXcds * ((direct.E + kXcds - 1) / kXcds) * n_ct : kXcds * xcd_tile_cap(mt_cap * n_ct),
+                  GATE_UP ? 1 : k_split);
   const TileDesc *tiles = GATE_UP ? d.tiles_gate_up : d.tiles_down;
   if (w_scale) {
-    grouped_gemm_kernel<C, GATE_UP, true, GATHER, DIRECT><<<grid, C::THREADS, 0, s>>>(
-        a, w, w_scale, ba, bb, tiles, d.totals, d.rowmap, out, K, N, limit, direct);
+    grouped_gemm_kernel<CF, GATE_UP, true, GATHER, DIRECT><<<grid, CF::THREADS, 0, s>>>(
+        a, w, w_scale, ba, bb, tiles, d.totals, d.rowmap, out, K, N, limit, direct, split_stride);
   } else {
     grouped_gemm_kernel<C, GATE_UP, false, GATHER, DIRECT><<<grid, C::THREADS, 0, s>>>(
-        a, w, nullptr, ba, bb, tiles, d.totals, d.rowmap, out, K, N, limit, direct);
+        a, w, nullptr, ba, bb, tiles, d.totals, d.rowmap, out, K, N, limit, direct, split_stride);
   }
   return hipGetLastError();
 }
@@ -971,26 +1011,33 @@ hipError_t launch_gate_up(const uint16_t *x, const void *w1, const uint16_t *w1_
   const uint4 *rows = reinterpret_cast<const uint4 *>(x);
   if (direct.topk_i)
     return launch_gemm<CfgGemmSmall, true, true, true>(rows, w, w1_scale, b1g, b1u, d, act, H, IM, limit,
-                                                       mt_cap, direct, s);
+                                                       mt_cap, direct, 1, 0, s);
   // either way the row operand is read from the token rows: 32 bytes of 32 rows per
   // instruction in the small-batch configuration, whole lines of 8 rows otherwise
   if (small_batch(max_rows))
     return launch_gemm<CfgGemmSmall, true, true>(rows, w, w1_scale, b1g, b1u, d, act, H, IM, limit, mt_cap,
-                                                 direct, s);
-  return launch_gemm<CfgGemm, true, true>(rows, w, w1_scale, b1g, b1u, d, act, H, IM, limit, mt_cap, direct, s);
+                                                 direct, 1, 0, s);
+  return launch_gemm<CfgGemm, true, true>(rows, w, w1_scale, b1g, b1u, d, act, H, IM, limit, mt_cap, direct, 1, 0,
+                                          s);
 }
 
 hipError_t launch_down(const uint16_t *act, const void *w2, const uint16_t *w2_scale, const float *b2,
                        const DispatchBuffers &d, float *y, int H, int IM, int mt_cap, int max_rows,
-                       const DirectIds &direct, hipStream_t s) {
+                       const DirectIds &direct, int k_split, size_t split_stride, hipStream_t s) {
   const uint4 *a = reinterpret_cast<const uint4 *>(act);
   const uint4 *w = reinterpret_cast<const uint4 *>(w2);
+  // The smallest batches: a workgroup is one stream of weights, and the few
+  // experts such a batch reaches leave most CUs without one.  Two workgroups
+  // per tile then sum half of the reduction each into their own copy of the
+  // rows (down_k_split; the combine adds the two parts).
+  const int ks = small_batch(max_rows) ? k_split : 1;
   if (direct.topk_i)
-    return launch_gemm<CfgGemmSmall, false, false, true>(a, w, w2_scale, b2, nullptr, d, y, IM, H, 0.f,
-                                                         mt_cap, direct, s);
+    return launch_gemm<CfgGemmSmall, false, false, true, CfgGemmSmallFp4>(a, w, w2_scale, b2, nullptr, d, y, IM, H,
+                                                                          0.f, mt_cap, direct, ks, split_stride, s);
   if (small_batch(max_rows))
-    return launch_gemm<CfgGemmSmall, false>(a, w, w2_scale, b2, nullptr, d, y, IM, H, 0.f, mt_cap, direct, s);
-  return launch_gemm<CfgGemm, false>(a, w, w2_scale, b2, nullptr, d, y, IM, H, 0.f, mt_cap, direct, s);
+    return launch_gemm<CfgGemmSmall, false, false, false, CfgGemmSmallFp4>(a, w, w2_scale, b2, nullptr, d, y, IM, H,
+                                                                           0.f, mt_cap, direct, ks, split_stride, s);
+  return launch_gemm<CfgGemm, false>(a, w, w2_scale, b2, nullptr, d, y, IM, H, 0.f, mt_cap, direct, 1, 0, s);
 }
 
 }  // namespace moe

@@ -73,7 +73,8 @@ struct moe_handle {
   DirectIds unplanned{nullptr, nullptr, 0, 0};
   // expert pipeline
   uint16_t *act = nullptr;  // SwiGLU output, bf16 fragments
-  float *y = nullptr;       // down output [a_pad_cap, H]
+  float *y = nullptr;       // down output [a_pad_cap, Hp], then the second part of a split reduction
+  int y_parts = 1;          // copies of y the last down GEMM wrote (down_k_split)
   uint16_t *t_norm = nullptr;  // normalised rows of moe_block_forward [max_tokens, H], allocated on first use
   uint16_t *x_pad = nullptr;   // the batch's rows widened to Hp columns [max_tokens, Hp]; only where Hp != H
 
@@ -159,7 +160,10 @@ int run_gemms(moe_handle *h, int layer, const uint16_t *x, int T, int max_rows, 
                          h->disp, h->act, h->Hp, h->IMp, c.swiglu_limit, mt_cap, max_rows, direct, s));
   HIP_TRY(tm.mark(MOE_STAGE_DOWN));
   HIP_TRY(launch_down(h->act, lw.w2q ? static_cast<const void *>(lw.w2q) : lw.w2, lw.w2s, lw.b2,
-                      h->disp, h->y, h->Hp, h->IMp, mt_cap, max_rows, direct, s));
+                      h->disp, h->y, h->Hp, h->IMp, mt_cap, max_rows, direct,
+                      down_k_split(max_rows, h->IMp, h->Hp, c.experts, T),
+                      (size_t)h->a_pad_cap * h->Hp * sizeof(float), s));
+  h->y_parts = down_k_split(max_rows, h->IMp, h->Hp, c.experts, T);
   return MOE_OK;
 }
 
@@ -169,9 +173,11 @@ int run_combine(moe_handle *h, const float *topk_v, const int *pos, int T, float
                 uint16_t *resid, const DirectIds &direct, hipStream_t s, StageTimer &tm) {
   HIP_TRY(tm.mark(MOE_STAGE_COMBINE));
   if (out) {
-    HIP_TRY(launch_combine(h->y, h->Hp, h->disp.inv, topk_v, pos, out, T, h->cfg.hidden, accumulate, direct, s));
+    HIP_TRY(launch_combine(h->y, h->Hp, h->y_parts, (size_t)h->a_pad_cap * h->Hp, h->disp.inv, topk_v, pos, out, T,
+                           h->cfg.hidden, accumulate, direct, s));
   } else {
-    HIP_TRY(launch_combine_residual(h->y, h->Hp, h->disp.inv, topk_v, pos, resid, T, h->cfg.hidden, direct, s));
+    HIP_TRY(launch_combine_residual(h->y, h->Hp, h->y_parts, (size_t)h->a_pad_cap * h->Hp, h->disp.inv, topk_v, pos,
+                                    resid, T, h->cfg.hidden, direct, s));
   }
   HIP_TRY(tm.mark(MOE_NUM_STAGES));
   return MOE_OK;
@@ -260,7 +266,8 @@ int moe_create(const moe_config *cfg, moe_handle **out) {
   ALLOC(h->disp.tiles_gate_up, (size_t)h->disp.tile_cap_gate_up);
   ALLOC(h->disp.tiles_down, (size_t)h->disp.tile_cap_down);
   ALLOC(h->act, (size_t)h->a_pad_cap * h->IMp);
-  ALLOC(h->y, (size_t)h->a_pad_cap * h->Hp);
+  // behind the rows of y: the second part of a split reduction (small batches, see down_k_split)
+  ALLOC(h->y, ((size_t)h->a_pad_cap + (kSmallBatchKSplit - 1) * small_batch_pad_rows(E)) * h->Hp);
   if (h->Hp != H) ALLOC(h->x_pad, (size_t)T * h->Hp);
 #undef ALLOC
   h->disp.a_pad_cap = h->a_pad_cap;

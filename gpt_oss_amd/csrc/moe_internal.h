@@ -174,20 +174,45 @@ inline bool direct_plan_fits(int T, int max_rows, int E, int a_pad_cap) {
 // run the small-batch configuration of both GEMMs.
 constexpr int kSmallBatchRows = 64;
 inline bool small_batch(int max_rows) { return max_rows <= kSmallBatchRows; }
+// Parts the down GEMM's reduction is split into (each part writes its own copy
+// of the output rows, which the combine adds up): two in the small-batch
+// configuration while the experts a batch of T tokens can reach have at most
+// one tile per CU between them -- a tile is one stream of weights there, and a
+// CU takes in two to three such streams at once --, else one.  Measured with
+// MXFP4 weights at 32 experts: a layer call at 1 token 54.8 -> 47.9 us, at 4
+// tokens 65 -> 62; from 8 tokens on the split gains nothing (the first GEMM's
+// workgroups already fill the CUs when the second starts).
+constexpr int kSmallBatchKSplit = 2;
+constexpr int kCus = 256;
+inline int down_k_split(int max_rows, int inter_padded, int hidden_padded, int E, int T) {
+  if (!small_batch(max_rows) || inter_padded < 64) return 1;
+  const int n_ct = (hidden_padded / kRowBlock + kGemmTileNb - 1) / kGemmTileNb;
+  const long long reach = (long long)T * kTopK < E ? (long long)T * kTopK : E;
+  return reach * n_ct <= kCus ? kSmallBatchKSplit : 1;
+}
+// The rows a small batch can reach in the padded row space: every expert's
+// rows rounded up to 32, or its fixed slot of 64 rows without a dispatch pass.
+inline int small_batch_pad_rows(int E) {
+  const int planned = kSmallBatchRows * kTopK + kTileGran * E, slots = kDirectSlotRows * E;
+  return planned > slots ? planned : slots;
+}
 hipError_t launch_gate_up(const uint16_t *x, const void *w1, const uint16_t *w1_scale, const float *b1g,
                           const float *b1u, const DispatchBuffers &d, uint16_t *act, int H, int IM,
                           float limit, int mt_cap, int max_rows, const DirectIds &direct, hipStream_t s);
+// k_split: parts of the reduction (down_k_split); split_stride: bytes between the copies of y they write
 hipError_t launch_down(const uint16_t *act, const void *w2, const uint16_t *w2_scale, const float *b2,
                        const DispatchBuffers &d, float *y, int H, int IM, int mt_cap, int max_rows,
-                       const DirectIds &direct, hipStream_t s);
+                       const DirectIds &direct, int k_split, size_t split_stride, hipStream_t s);
 // direct.topk_i != nullptr: the rows of y are found from the ids (inv is not read)
-// ldy: floats per row of y (the padded hidden size)
-hipError_t launch_combine(const float *y, int ldy, const int *inv, const float *topk_v, const int *pos,
-                          float *out, int T, int H, int accumulate, const DirectIds &direct,
-                          hipStream_t s);
-hipError_t launch_combine_residual(const float *y, int ldy, const int *inv, const float *topk_v,
-                                   const int *pos, uint16_t *x, int T, int H, const DirectIds &direct,
-                                   hipStream_t s);
+// ldy: floats per row of y (the padded hidden size).  y_parts copies of y lie
+// part_stride floats apart (the parts of a split reduction, see down_k_split);
+// a row of the down projection is their sum, added in that order.
+hipError_t launch_combine(const float *y, int ldy, int y_parts, size_t part_stride, const int *inv,
+                          const float *topk_v, const int *pos, float *out, int T, int H, int accumulate,
+                          const DirectIds &direct, hipStream_t s);
+hipError_t launch_combine_residual(const float *y, int ldy, int y_parts, size_t part_stride, const int *inv,
+                                   const float *topk_v, const int *pos, uint16_t *x, int T, int H,
+                                   const DirectIds &direct, hipStream_t s);
 hipError_t launch_rmsnorm(const uint16_t *x, const float *weight, const int *pos, uint16_t *t_out,
                           int T, int H, hipStream_t s);
 

@@ -314,15 +314,18 @@ def test_all_tokens_on_four_experts_and_tiny_batches(c2):
         check_outputs(R, L2, x, None, np.arange(T))
 
 
-@pytest.mark.parametrize("T", [16, 17, 64, 65, 128, 129, 256, 257])
+@pytest.mark.parametrize("T", [5, 6, 16, 17, 64, 65, 128, 129, 256, 257])
 def test_batch_size_boundaries(c2, T):
     """Either side of the sizes at which the library changes its plan: up to 64
     rows per expert the GEMMs run in their small-batch configuration and gate_up
     reads the token rows itself, up to 128 tokens several workgroups share a
-    router tile, up to 256 tokens the dispatch is one workgroup.
+    router tile, up to 256 tokens the dispatch is one workgroup, up to 5 tokens
+    (at 32 experts and 12 column tiles) the down GEMM's reduction is split over
+    two workgroups per tile.
     moe_forward bounds the rows per expert by T, moe_experts (whose ids come from
-    the caller) by 4 T, so between 17 and 64 tokens the two entry points take
-    different configurations for the same work: same bits required."""
+    the caller) by 4 T unless the caller promises distinct ids, so between 17
+    and 64 tokens the two entry points take different configurations for the
+    same work: same bits required, with the promise and without."""
     sh, L, m = c2
     x = L["x"][500:500 + T]
     R = abi.run_layer(m, 0, x, None)
@@ -331,9 +334,17 @@ def test_batch_size_boundaries(c2, T):
     dx = abi.DevBuf.from_numpy(synth.to_bf16_bits(x))
     dti, dtv = abi.DevBuf.from_numpy(R["topk_i"]), abi.DevBuf.from_numpy(R["topk_v"])
     dout = abi.DevBuf(T * sh.hidden * 4)
-    m.experts(0, dx, None, dti, dtv, T, dout, accumulate=False)
-    abi.sync()
-    assert np.array_equal(dout.download((T, sh.hidden), np.float32), R["out"])
+    try:
+        for distinct in (True, False):
+            m.set_distinct_ids(distinct)
+            m.experts(0, dx, None, dti, dtv, T, dout, accumulate=False)
+            abi.sync()
+            got = dout.download((T, sh.hidden), np.float32)
+            # (at this shape only batches of up to 5 tokens split the reduction, and those run the
+            # small-batch configuration with or without the promise)
+            assert np.array_equal(got, R["out"]), f"distinct={distinct}"
+    finally:
+        m.set_distinct_ids(False)
 
 
 def test_c4_120b_shape():
@@ -407,6 +418,7 @@ def test_small_batches_without_dispatch_pass(c2, T):
     x = L["x"][900:900 + T]
     pos = np.where(np.random.default_rng(T).random(T) < 0.3, -1, 3).astype(np.int32)
     pos[0] = 3
+    m.set_distinct_ids(True)  # the staged calls then run the small-batch configuration up to 64 tokens, too
     for p in (None, pos):
         R = abi.run_layer(m, 0, x, p)
         check_routing(R, L, x, p, sh.experts)
@@ -431,6 +443,7 @@ def test_small_batches_without_dispatch_pass(c2, T):
     m.forward(0, dx, dpos, T, dout, accumulate=True)
     abi.sync()
     got = dout.download((T, H), np.float32)
+    m.set_distinct_ids(False)
     assert np.array_equal(got[pos < 0], prior[pos < 0])
     np.testing.assert_allclose(got[pos >= 0], prior[pos >= 0] + a[pos >= 0], rtol=0, atol=1e-6)
 
