@@ -395,3 +395,51 @@ def test_large_batches_repeat_bit_for_bit():
         if ref is None:
             ref = got
         assert np.array_equal(got, ref), f"FFN block, call {i}: other bits"
+
+
+# ---------------- HIP-graph replay of the paths added later ----------------
+
+@pytest.mark.parametrize("T", [3, 100])
+def test_padded_shape_and_split_reduction_replay_from_a_hip_graph(T):
+    """moe_forward at a hidden size that needs padding (one more kernel per call,
+    the row widening) and, at 3 tokens, with the down GEMM's reduction split over
+    two workgroups per tile: captured once, replayed three times with eager
+    calls of another size in between, every replay bit-identical to the eager
+    result."""
+    import ctypes as C
+    hip = C.CDLL("libamdhip64.so")
+
+    def ok(rc):
+        assert rc == 0, f"HIP call failed with {rc}"
+
+    sh = synth.LayerShape("g", T, 96, 96, 8)
+    L = bf16_layer(sh, seed=13)
+    m = make_moe(sh, L, 128)
+    H = sh.hidden
+    dx = abi.DevBuf.from_numpy(synth.to_bf16_bits(L["x"]))
+    dout, dref = abi.DevBuf(T * H * 4), abi.DevBuf(T * H * 4)
+    stream = C.c_void_p()
+    ok(hip.hipStreamCreate(C.byref(stream)))
+    m.forward(0, dx, None, T, dref, stream=stream)
+    ok(hip.hipStreamSynchronize(stream))
+    ref = dref.download((T, H), np.float32)
+    want = ob.moe_layer(L["x"], None, *[L[k] for k in W], 4, sh.limit, mode=ob.ROUND_ACT_BF16 | ob.PAR_TOKENS)
+    assert np.abs(ref - want).max() <= 2e-2 and np.linalg.norm(ref - want) <= 1e-3 * np.linalg.norm(want)
+    graph, gexec = C.c_void_p(), C.c_void_p()
+    ok(hip.hipStreamBeginCapture(stream, C.c_int(0)))
+    m.forward(0, dx, None, T, dout, stream=stream)
+    ok(hip.hipStreamEndCapture(stream, C.byref(graph)))
+    ok(hip.hipGraphInstantiate(C.byref(gexec), graph, None, None, C.c_size_t(0)))
+    try:
+        for _ in range(3):
+            dout.memset(0)
+            abi.sync()
+            ok(hip.hipGraphLaunch(gexec, stream))
+            ok(hip.hipStreamSynchronize(stream))
+            assert np.array_equal(dout.download((T, H), np.float32), ref)
+            m.forward(0, dx, None, max(T // 2, 1), dref, stream=stream)  # eager work of another size
+            ok(hip.hipStreamSynchronize(stream))
+    finally:
+        hip.hipGraphExecDestroy(gexec)
+        hip.hipGraphDestroy(graph)
+        hip.hipStreamDestroy(stream)
