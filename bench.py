@@ -121,7 +121,7 @@ def cpu_baseline(shape, L, budget_s=12.0):
     return out
 
 
-def run_leg(shape, steps, warmup, device_timed=False, mxfp4=None):
+def run_leg(shape, steps, warmup, device_timed=False, mxfp4=None, zero_expert_weights=False):
     """Uploads the workload's layer, runs `warmup` + `steps` forwards and returns
     (seconds per step, stage times in ms from HIP events in the timed steps,
     calls measured, median seconds per step, host-side layer or None).  Seconds
@@ -129,7 +129,10 @@ def run_leg(shape, steps, warmup, device_timed=False, mxfp4=None):
     device_timed takes them from two HIP events around the steps enqueued by one
     library call instead (a step of 150 us is otherwise timed by the
     interpreter's call overhead).  The median is over per-step HIP-event
-    intervals of a further run of max(steps, 50) steps."""
+    intervals of a further run of max(steps, 50) steps.  zero_expert_weights: a
+    yardstick, not a workload -- the expert matrices and biases are uploaded as
+    zeros (router, routing, tile plan, instructions and memory traffic are those
+    of the workload; what changes is how many bits toggle in the matrix cores)."""
     from gpt_oss_amd import abi, synth
     T, H, IM, E = shape.tokens, shape.hidden, shape.inter, shape.experts
     moe = abi.Moe(H, IM, E, max_tokens=T, swiglu_limit=shape.limit)
@@ -143,6 +146,9 @@ def run_leg(shape, steps, warmup, device_timed=False, mxfp4=None):
         x = synth.make_activations(shape)
     else:
         L = synth.make_layer(shape, seed=0)
+        if zero_expert_weights:
+            for k in ("w_mlp1", "b_mlp1", "w_mlp2", "b_mlp2"):
+                L[k][...] = 0
         moe.upload_layer(0, *[L[k] for k in ("w_router", "b_router", "w_mlp1", "b_mlp1", "w_mlp2", "b_mlp2")])
         x = L["x"]
     dx = abi.DevBuf.from_numpy(synth.to_bf16_bits(x))
@@ -216,6 +222,9 @@ def main():
     ap.add_argument("--workload", default="c2",
                     help="c2 (headline), c3a, c3b, c4, c5 (MXFP4 decode); d4: yardstick, four dense GEMMs of 4096 rows")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--zero-expert-weights", action="store_true",
+                    help="yardstick, bf16 workloads only: the expert matrices are uploaded as zeros (same routing, "
+                         "tiles, instructions and traffic; the line is marked and is not a benchmark result)")
     ap.add_argument("--no-decode", action="store_true",
                     help="c2 only: skip the side figures (MXFP4 weights: workload c5 and c2's batch; "
                          "the other configurations c3a, c3b, c4)")
@@ -233,7 +242,13 @@ def main():
     shape = synth.CONFIGS[args.workload]
     T, H, IM, E, K = shape.tokens, shape.hidden, shape.inter, shape.experts, shape.topk
     mxfp4 = shape.name == "c5"
-    s_per_step, stages, n_meas, median_s, L = run_leg(shape, args.steps, args.warmup)
+    if args.zero_expert_weights:
+        if mxfp4:
+            print("--zero-expert-weights is for the bf16 workloads", file=sys.stderr)
+            sys.exit(2)
+        args.no_decode = args.no_cpu_baseline = True  # a yardstick line carries neither
+    s_per_step, stages, n_meas, median_s, L = run_leg(shape, args.steps, args.warmup,
+                                                      zero_expert_weights=args.zero_expert_weights)
 
     A = T * K
     flops_gate_up = 2.0 * A * H * 2 * IM
@@ -288,6 +303,8 @@ def main():
     roofline["frac_mfma_peak"] = mfma_tflops / PEAK_BF16_TFLOPS
     roofline["frac_hbm_peak"] = hbm_gbs / PEAK_HBM_GBS
     weights = "MXFP4 expert weights" if mxfp4 else "bf16 weights"
+    if args.zero_expert_weights:
+        weights = "bf16 weights ALL ZERO (yardstick: not a benchmark result)"
     result = {
         "metric": "MoE-layer tokens/sec",
         "value": T / s_per_step,
