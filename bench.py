@@ -12,7 +12,10 @@ line also carries "decode_mxfp4", a side figure for the decode-regime
 configuration (64 tokens, MXFP4 expert weights; `--workload c5` makes that
 configuration the one measured), "prefill_mxfp4", the headline batch with
 MXFP4 expert weights, and "other_workloads", short legs of the remaining
-benchmark configurations (c3a, c3b, c4).  None of them is part of `value`.
+benchmark configurations (c3a, c3b, c4), and "zero_weights_yardstick", the
+headline workload once more with all-zero expert matrices (the same kernels at
+the clock the GPU holds when their operands do not toggle).  None of them is
+part of `value`.
 """
 from __future__ import annotations
 
@@ -121,7 +124,7 @@ def cpu_baseline(shape, L, budget_s=12.0):
     return out
 
 
-def run_leg(shape, steps, warmup, device_timed=False, mxfp4=None, zero_expert_weights=False):
+def run_leg(shape, steps, warmup, device_timed=False, mxfp4=None, zero_expert_weights=False, layer=None):
     """Uploads the workload's layer, runs `warmup` + `steps` forwards and returns
     (seconds per step, stage times in ms from HIP events in the timed steps,
     calls measured, median seconds per step, host-side layer or None).  Seconds
@@ -132,7 +135,9 @@ def run_leg(shape, steps, warmup, device_timed=False, mxfp4=None, zero_expert_we
     intervals of a further run of max(steps, 50) steps.  zero_expert_weights: a
     yardstick, not a workload -- the expert matrices and biases are uploaded as
     zeros (router, routing, tile plan, instructions and memory traffic are those
-    of the workload; what changes is how many bits toggle in the matrix cores)."""
+    of the workload; what changes is how many bits toggle in the matrix cores).
+    layer: a host-side layer of this shape to use instead of generating one (it
+    is zeroed in place when zero_expert_weights is set)."""
     from gpt_oss_amd import abi, synth
     T, H, IM, E = shape.tokens, shape.hidden, shape.inter, shape.experts
     moe = abi.Moe(H, IM, E, max_tokens=T, swiglu_limit=shape.limit)
@@ -145,7 +150,7 @@ def run_leg(shape, steps, warmup, device_timed=False, mxfp4=None, zero_expert_we
         moe.upload_layer_mxfp4(0, wr, br, b1k, s1, b1, b2k, s2, b2)
         x = synth.make_activations(shape)
     else:
-        L = synth.make_layer(shape, seed=0)
+        L = layer if layer is not None else synth.make_layer(shape, seed=0)
         if zero_expert_weights:
             for k in ("w_mlp1", "b_mlp1", "w_mlp2", "b_mlp2"):
                 L[k][...] = 0
@@ -367,6 +372,20 @@ def main():
         result["other_workloads"] = {n: side_leg(n) for n in ("c3a", "c3b", "c4")}
     if not args.no_cpu_baseline and L is not None:
         result["cpu_baseline"] = cpu_baseline(shape, L)
+    if shape.name == "c2" and not args.no_decode and L is not None:
+        # Yardstick, not a result: the headline workload once more with the expert
+        # matrices uploaded as zeros -- same routing, tiles, instructions and memory
+        # traffic; the matrix cores' operands stop toggling and the GPU holds a
+        # higher clock.  Says how much of the distance to the published peak is
+        # the clock under load and how much the kernels' idle cycles.
+        _, stz, _, _, _ = run_leg(shape, 60, 10, zero_expert_weights=True, layer=L)
+        tg, td = stz["gate_up"] * 1e-3, stz["down"] * 1e-3
+        result["zero_weights_yardstick"] = {
+            "workload": "c2 with all-zero expert weights (not a benchmark result)",
+            "stage_us": {k: v * 1e3 for k, v in stz.items()},
+            "gate_up_tflops": flops_gate_up / tg / 1e12,
+            "gate_up_frac_bf16_peak": flops_gate_up / tg / 1e12 / PEAK_BF16_TFLOPS,
+            "expert_gemms_frac_bf16_peak": (flops_gate_up + flops_down) / (tg + td) / 1e12 / PEAK_BF16_TFLOPS}
     print(json.dumps(result))
 
 
